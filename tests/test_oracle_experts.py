@@ -1,0 +1,92 @@
+"""Pins the floating-point oracle against independent statements of the same
+mathematics: a dense all-experts evaluation, the textbook SwiGLU MLP, autograd
+in fp64, and torch.autograd.gradcheck."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from helpers import make_layer_inputs
+
+
+def test_forward_matches_dense_evaluation():
+    x, W1, W2, mask, s, _ = make_layer_inputs(40, 16, 8, 6, 3, seed=1)
+    y = oracle.experts_forward(x, W1, W2, mask, s, dtype=torch.float64)
+    yd = oracle.experts_forward_dense(x, W1, W2, mask, s)
+    torch.testing.assert_close(y, yd, rtol=1e-12, atol=1e-12)
+
+
+def test_single_expert_is_plain_swiglu_mlp():
+    # N=1, K=1, s=1: y = (up(x) * silu(gate(x))) @ down, with up = first H columns
+    # and gate = last H columns of Wl1 (the activation is on the SECOND half).
+    torch.manual_seed(0)
+    M, D, H = 12, 10, 6
+    x = torch.randn(M, D, dtype=torch.float64)
+    W1 = torch.randn(1, D, 2 * H, dtype=torch.float64)
+    W2 = torch.randn(1, H, D, dtype=torch.float64)
+    mask = torch.ones(1, M, dtype=torch.int32)
+    s = torch.ones(1, M)
+    y = oracle.experts_forward(x, W1, W2, mask, s, dtype=torch.float64)
+    up = F.linear(x, W1[0, :, :H].T)
+    gate = F.linear(x, W1[0, :, H:].T)
+    ref = F.linear(up * F.silu(gate), W2[0].T)
+    torch.testing.assert_close(y, ref, rtol=1e-12, atol=1e-12)
+    # swapping the halves must change the result (guards the half order)
+    W1s = torch.cat([W1[..., H:], W1[..., :H]], dim=-1)
+    assert not torch.allclose(oracle.experts_forward(x, W1s, W2, mask, s, dtype=torch.float64), ref)
+
+
+def test_linearity_in_gate_weights():
+    x, W1, W2, mask, s, _ = make_layer_inputs(24, 8, 4, 5, 2, seed=2)
+    s = s.double()
+    y1 = oracle.experts_forward(x, W1, W2, mask, s, dtype=torch.float64)
+    y2 = oracle.experts_forward(x, W1, W2, mask, 3.0 * s, dtype=torch.float64)
+    torch.testing.assert_close(3.0 * y1, y2, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("Ks", [0, 2])
+def test_closed_form_backward_matches_autograd(Ks):
+    M, D, H, N, K = 48, 16, 8, 6, 3
+    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, Ks=Ks, seed=4, wstd=0.3)
+    xs = x.double().requires_grad_()
+    W1d = W1.double().requires_grad_()
+    W2d = W2.double().requires_grad_()
+    sd = s.double().clone().requires_grad_()
+    y = oracle.experts_forward(xs, W1d, W2d, mask, sd, dtype=torch.float64)
+    y.backward(dy.double())
+    G_x, G_W1, G_W2, G_s = oracle.experts_backward_closed_form(x, W1, W2, mask, s, dy)
+    torch.testing.assert_close(G_x, xs.grad, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(G_W1, W1d.grad, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(G_W2, W2d.grad, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(G_s, sd.grad, rtol=1e-10, atol=1e-10)
+    # off-mask entries of G_s are exactly zero
+    assert torch.all(G_s[mask == 0] == 0)
+
+
+def test_gradcheck_fp64():
+    M, D, H, N, K = 6, 4, 3, 3, 2
+    x, W1, W2, mask, s, _ = make_layer_inputs(M, D, H, N, K, seed=6, wstd=0.5)
+    args = [t.double().clone().requires_grad_() for t in (x, W1, W2, s)]
+    fn = lambda x_, a_, b_, s_: oracle.experts_forward(x_, a_, b_, mask, s_, dtype=torch.float64)
+    assert torch.autograd.gradcheck(fn, args, eps=1e-6, atol=1e-5)
+
+
+def test_expert_without_tokens_gets_zero_weight_grads():
+    M, D, H, N = 10, 4, 3, 3
+    torch.manual_seed(1)
+    x, dy = torch.randn(M, D), torch.randn(M, D)
+    W1, W2 = torch.randn(N, D, 2 * H), torch.randn(N, H, D)
+    mask = torch.zeros(N, M, dtype=torch.int32)
+    mask[0] = 1
+    mask[2] = 1
+    s = torch.rand(N, M) * mask
+    _, G_W1, G_W2, _ = oracle.experts_backward_closed_form(x, W1, W2, mask, s, dy)
+    assert torch.all(G_W1[1] == 0) and torch.all(G_W2[1] == 0)
+
+
+def test_module_signature_and_outputs():
+    M, D, H, N, K = 32, 8, 4, 4, 2
+    x, W1, W2, mask, s, _ = make_layer_inputs(M, D, H, N, K, seed=7)
+    m = oracle.OracleMoMoE(D, H, N, K, save_percent=0, Wl1_ND2H=W1, Wl2_NHD=W2)
+    y, sizes = m(x.reshape(2, 16, D), mask, s)
+    assert y.shape == (2, 16, D) and sizes.dtype == torch.int64 and sizes.sum() == M * K
