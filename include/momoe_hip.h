@@ -1,0 +1,174 @@
+/* C ABI of libmomoe_hip.so: hand-written gfx950 (MI355X) kernels for the MoMoE
+ * SwiGLU mixture-of-experts layer.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is DEVICE memory unless said
+ *     otherwise; bf16 tensors are passed as `void*`/`const void*`.
+ *   - nothing is allocated or freed; the caller owns every buffer and sizes the
+ *     workspaces with the *_ints / *_bytes queries below.
+ *   - work is only ENQUEUED on `stream` (a hipStream_t passed as void*); no entry
+ *     point synchronises with the device.
+ *   - the return value is a status code (MOMOE_OK or MOMOE_ERR_*); no C++
+ *     exception crosses the boundary.  Entry points are re-entrant and keep no
+ *     global mutable state.
+ *   - dimension letters: M tokens, D embedding, H expert hidden, N experts,
+ *     K experts per token, Msum = M*K (token,expert) pairs = "sorted rows":
+ *     the rows of expert i occupy [cumsums[i], cumsums[i+1]) in ascending token order.
+ *
+ * Each declaration cites the part of the reference (tilde-research/MoMoE-impl,
+ * paths relative to its root) that it replaces.
+ */
+#ifndef MOMOE_HIP_H
+#define MOMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOMOE_OK 0
+#define MOMOE_ERR_BAD_ARG 1     /* null pointer, negative size, misaligned pointer */
+#define MOMOE_ERR_UNSUPPORTED 2 /* shape outside what the kernels handle */
+#define MOMOE_ERR_LAUNCH 3      /* the HIP runtime refused a launch */
+
+/* rows per row-tile of the grouped GEMMs; the tile table must be built with it */
+#define MOMOE_TILE_ROWS 128
+/* column-block width of the partial row sums written by momoe_dgrad_h_swiglu_bwd */
+#define MOMOE_GS_BLOCK 256
+
+int momoe_abi_version(void);
+const char* momoe_status_string(int status);
+
+/* ---- routing index -------------------------------------------------------
+ * Replaces find_used_experts + scatter_cols_kernel (momoe/momoe.py:821-842,
+ * 760-815) and the torch.sum at :830.
+ *
+ * mask_NM: int32 0/1, element (i,m) at mask[i*stride_n + m*stride_m].
+ * Outputs: sizes_N int64[N]; cumsums_N1 int32[N+1]; idx_Msum int32[M*K]
+ * (token of each sorted row); which_Msum int32[M*K] (slot of the pair within its
+ * token = number of lower-numbered experts holding the token); inv_MK
+ * int32[M*K] (sorted row of token m's k-th pair); tile_table
+ * int32[momoe_tile_table_ints()] (device-side list of (expert,row-block) tiles
+ * so that no GEMM launch depends on host knowledge of the routing);
+ * violations int32[1] += number of tokens whose pair count differs from K
+ * (caller zeroes it; if the total pair count exceeds M*K the tile table is
+ * emptied so later kernels touch nothing).
+ */
+int64_t momoe_tile_table_ints(int64_t M, int64_t N, int64_t K, int tile_rows);
+int64_t momoe_index_workspace_bytes(int64_t M, int64_t N);
+int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m,
+                      int64_t M, int64_t N, int64_t K,
+                      int64_t* sizes_N, int32_t* cumsums_N1, int32_t* idx_Msum,
+                      int32_t* which_Msum, int32_t* inv_MK,
+                      int32_t* tile_table, int tile_rows,
+                      void* workspace, int64_t workspace_bytes,
+                      int32_t* violations, void* stream);
+
+/* ---- experts forward -----------------------------------------------------
+ * momoe_lin1_swiglu_fwd replaces lin1_kernel (momoe/momoe.py:69-152):
+ *   [a|b] = x[idx[r]] @ Wl1[i]  (fp32 accumulate), h[r] = bf16(a * b * sigmoid(b)).
+ * x_MD bf16 [M,D]; Wl1_ND2H bf16 [N,D,2H]; h_MsumH bf16 [Msum,H] (may be NULL:
+ * then only a|b is produced and row tiles entirely below ab_row_lo are skipped);
+ * ab_rows bf16 [*,2H] indexed by the sorted row r (may be NULL): rows with
+ * ab_row_lo <= r < ab_row_hi receive bf16(a)|bf16(b) (the selective save of
+ * :141-145 with lo=0, hi=Msave; the backward recomputation with lo=Msave, hi=Msum).
+ */
+int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
+                          const int32_t* tile_table, void* h_MsumH,
+                          void* ab_rows, int64_t ab_row_lo, int64_t ab_row_hi,
+                          int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+
+/* momoe_lin2_scale_fwd replaces lin2_kernel (momoe/momoe.py:161-237):
+ *   ys[r] = bf16( (h[r] @ Wl2[i]) * s[i, idx[r]] ), rows kept in sorted order.
+ * s_NM fp32, element (i,m) at s[i*s_stride_n + m*s_stride_m]. ys_MsumD bf16 [Msum,D].
+ */
+int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD,
+                         const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
+                         const int32_t* idx_Msum, const int32_t* tile_table, void* ys_MsumD,
+                         int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+
+/* momoe_combine replaces y_KMD.sum(dim=0) / G_x_KMD.sum(dim=0) (momoe/momoe.py:290, :754):
+ *   out[m] = bf16( sum_k rows[inv[m,k]] ) with fp32 accumulation, k ascending.
+ */
+int momoe_combine(const void* rows_MsumD, const int32_t* inv_MK, void* out_MD,
+                  int64_t M, int64_t D, int64_t K, int64_t Msum, void* stream);
+
+/* ---- experts backward ----------------------------------------------------
+ * momoe_dgrad_h_swiglu_bwd replaces making_nice_scatter_kernel (G_y part) and
+ * swiglu_backward_kernel (momoe/momoe.py:298-350, 421-535), and produces the
+ * gate-weight gradient that lin1_backward_kernel (:683-703) obtains from a
+ * recomputed down projection:
+ *   u    = G_y[idx[r]] @ Wl2[i]^T                      (fp32 accumulate over D)
+ *   a,b  = row r of ab_save (r < Msave) or of gz (r >= Msave, written there
+ *          beforehand by momoe_lin1_swiglu_fwd)
+ *   G_h  = s[i,idx[r]] * u
+ *   gz[r] = bf16( G_h*b*sig(b) | G_h*a*sig(b)*(1 + b*(1-sig(b))) )   (overwrites a|b)
+ *   hs[r] = bf16( s * a*b*sig(b) )       (h pre-scaled by the gate weight for the Wl2 gradient)
+ *   gs_part[p][r] = sum over the p-th block of MOMOE_GS_BLOCK hidden columns of u * a*b*sig(b)
+ * (sum_p gs_part[p][r] = G_y[idx[r]] . (h[r] @ Wl2[i]) = dL/ds, by associativity).
+ * gs_part fp32 [ceil(H/MOMOE_GS_BLOCK)][Msum].
+ */
+int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD,
+                             const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
+                             const int32_t* idx_Msum, const int32_t* tile_table,
+                             const void* ab_save, int64_t Msave,
+                             void* gz_Msum2H, void* hs_MsumH, float* gs_part,
+                             int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+
+/* momoe_gs_scatter: Gs_NM[i, idx[r]] = sum_p gs_part[p][r] for every sorted row r of
+ * expert i (momoe/momoe.py:699-703 without atomics).  Gs_NM fp32 contiguous [N,M],
+ * zero-filled by the caller (:721).
+ */
+int momoe_gs_scatter(const float* gs_part, int64_t nparts, const int32_t* idx_Msum,
+                     const int32_t* cumsums_N1, float* Gs_NM,
+                     int64_t M, int64_t N, int64_t Msum, void* stream);
+
+/* momoe_dgrad_x replaces the GEMM of lin1_backward_kernel (momoe/momoe.py:662-681):
+ *   gxs[r] = bf16( gz[r] @ Wl1[i]^T ), rows kept in sorted order; follow with
+ *   momoe_combine to obtain G_x.
+ */
+int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* tile_table,
+                  void* gxs_MsumD, int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum,
+                  void* stream);
+
+/* momoe_wgrad replaces weights_update_kernel (momoe/momoe.py:356-412):
+ *   GW[i][x][y] = bf16( sum over sorted rows r of expert i of A[ra(r)][x] * B[rb(r)][y] )
+ * with ra(r) = a_gather ? a_gather[r] : r (same for rb).  A bf16 with row stride lda
+ * (>= X), B bf16 with row stride ldb (>= Y).  Experts without rows get exact zeros.
+ * Wl2 gradient: A = hs (X=H), B = G_y gathered by idx (Y=D).
+ * Wl1 gradient: A = x gathered by idx (X=D), B = gz (Y=2H).
+ */
+int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
+                const void* B_rows, int64_t ldb, const int32_t* b_gather,
+                const int32_t* cumsums_N1, void* GW_NXY,
+                int64_t N, int64_t X, int64_t Y, int64_t Msum, void* stream);
+
+/* ---- router ----------------------------------------------------------------
+ * momoe_router_fwd replaces the elementwise part of TopKRouterFunction.forward
+ * (momoe/topk_router.py:96-120), given the gate logits (the matmul of :95 stays a
+ * library GEMM): fp32 softmax over the N-Ks routed and the Ks shared columns,
+ * top-(K-Ks) of (probability + bias) with ties going to the lower index,
+ * renormalisation.  logits_MN [M,N] row-major, bf16 (logits_f32=0) or fp32 (=1).
+ * Outputs: mask_NM int32 [N,M] contiguous; s_MN fp32 [M,N] (its transpose view is
+ * s_NM); p_sel_MN fp32 [M,N] (masked softmax probabilities, :106); Ng_M, Ks_M fp32 [M].
+ */
+int momoe_router_fwd(const void* logits_MN, int logits_f32, const float* biases_N,
+                     int64_t M, int64_t N, int64_t K, int64_t Ks,
+                     int32_t* mask_NM, float* s_MN, float* p_sel_MN, float* Ng_M, float* Ks_M,
+                     void* stream);
+
+/* momoe_router_bwd replaces normalize_backward_kernel (momoe/topk_router.py:11-56):
+ * gradient w.r.t. the gate logits, bf16 [M,N] row-major.  Gs_NM fp32, element (i,m) at
+ * Gs[i*gs_stride_n + m*gs_stride_m]; it is not modified.
+ */
+int momoe_router_bwd(const float* Gs_NM, int64_t gs_stride_n, int64_t gs_stride_m,
+                     const float* p_sel_MN, const float* s_MN, const float* Ng_M, const float* Ks_M,
+                     const int32_t* mask_NM, int64_t M, int64_t N, int64_t Ks,
+                     void* Glogits_MN, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOMOE_HIP_H */

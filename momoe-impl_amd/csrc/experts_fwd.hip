@@ -1,0 +1,226 @@
+// Forward of the experts: grouped GEMM x.Wl1 with fused SwiGLU, grouped GEMM
+// h.Wl2 with the gate weight fused into the epilogue, and the K-way combine.
+#include "gemm_tile.hpp"
+
+namespace momoe {
+namespace {
+
+constexpr int BM = MOMOE_TILE_ROWS;  // 128 sorted rows per tile
+constexpr int BN = 256;              // output columns per tile
+constexpr int FM = 2, FN = 4;        // 2x2 waves, each 64 rows x 128 columns
+
+struct Lin1Args {
+  const bf16* x;
+  const bf16* w1;
+  const int32_t* idx;
+  const int32_t* table;
+  bf16* h;
+  bf16* ab;
+  int64_t ab_lo, ab_hi;
+  int D, H;
+};
+
+// Tile = 128 rows x (128 `a` columns + the matching 128 `b` columns) so the SwiGLU
+// product pairs registers of the same lane.
+__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
+  using AOp = ROperand<BM>;
+  using BOp = TOperand<BN>;
+  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  constexpr int BNH = BN / 2;
+  const int nb = (p.H + BNH - 1) / BNH;
+  const TileCoord tc = decode_tile(p.table, nb);
+  if (!tc.valid) return;
+  if (p.h == nullptr && (int64_t)tc.row0 + tc.rows <= p.ab_lo) return;
+  const int j0 = tc.tn * BNH;
+  const int D = p.D, H = p.H;
+  const bf16* w = p.w1 + (int64_t)tc.expert * D * 2 * H;
+
+  AOp A;
+  BOp B;
+  A.init([&](int r) {
+    const int rr = min(r, tc.rows - 1);
+    return p.x + (int64_t)p.idx[tc.row0 + rr] * D;
+  });
+  B.init([&](int c) -> const bf16* {
+    const int half = c / BNH, j = j0 + (c % BNH);
+    return j < H ? w + half * H + j : nullptr;
+  }, 2 * H);
+
+  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
+  const int m_org[FM] = {wm * 64, wm * 64 + 32};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32, BNH + wn * 64, BNH + wn * 64 + 32};
+  f32x16 acc[FN][FM];
+  zero_acc<FM, FN>(acc);
+  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, D / kBK, lds, m_org, n_org);
+
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int rloc = m_org[i] + acc_row();
+    if (rloc >= tc.rows) continue;
+    const int64_t r = (int64_t)tc.row0 + rloc;
+    const bool save = p.ab != nullptr && r >= p.ab_lo && r < p.ab_hi;
+#pragma unroll
+    for (int f = 0; f < FN / 2; ++f) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int j = j0 + wn * 64 + f * 32 + acc_col(q);
+        if (j >= H) continue;
+        float a[4], b[4], hv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = acc[f][i][4 * q + e];
+          b[e] = acc[f + FN / 2][i][4 * q + e];
+          hv[e] = a[e] * b[e] * sigmoidf_fast(b[e]);
+        }
+        if (p.h) store_bf16x4(p.h + r * H + j, hv[0], hv[1], hv[2], hv[3]);
+        if (save) {
+          store_bf16x4(p.ab + r * 2 * H + j, a[0], a[1], a[2], a[3]);
+          store_bf16x4(p.ab + r * 2 * H + H + j, b[0], b[1], b[2], b[3]);
+        }
+      }
+    }
+  }
+}
+
+struct Lin2Args {
+  const bf16* h;
+  const bf16* w2;
+  const float* s;
+  int64_t ssn, ssm;
+  const int32_t* idx;
+  const int32_t* table;
+  bf16* ys;
+  int D, H;
+};
+
+__global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
+  using AOp = ROperand<BM>;
+  using BOp = TOperand<BN>;
+  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  const int D = p.D, H = p.H;
+  const int nb = (D + BN - 1) / BN;
+  const TileCoord tc = decode_tile(p.table, nb);
+  if (!tc.valid) return;
+  const int d0 = tc.tn * BN;
+  const bf16* w = p.w2 + (int64_t)tc.expert * H * D;
+
+  AOp A;
+  BOp B;
+  A.init([&](int r) { return p.h + ((int64_t)tc.row0 + min(r, tc.rows - 1)) * H; });
+  B.init([&](int c) -> const bf16* { return d0 + c < D ? w + d0 + c : nullptr; }, D);
+
+  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
+  const int m_org[FM] = {wm * 64, wm * 64 + 32};
+  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
+  f32x16 acc[FN][FM];
+  zero_acc<FM, FN>(acc);
+  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, H / kBK, lds, m_org, n_org);
+
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int rloc = m_org[i] + acc_row();
+    if (rloc >= tc.rows) continue;
+    const int64_t r = (int64_t)tc.row0 + rloc;
+    const float sv = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[r] * p.ssm];
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int d = d0 + n_org[f] + acc_col(q);
+        if (d >= D) continue;
+        store_bf16x4(p.ys + r * D + d, acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
+                     acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv);
+      }
+    }
+  }
+}
+
+// out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.
+__global__ __launch_bounds__(256) void combine_kernel(const bf16* __restrict__ rows,
+                                                      const int32_t* __restrict__ inv,
+                                                      bf16* __restrict__ out, int D, int K,
+                                                      int64_t msum) {
+  const int64_t m = blockIdx.x;
+  for (int c = threadIdx.x; c < D / 8; c += blockDim.x) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < K; ++k) {
+      const int32_t r = inv[m * K + k];
+      if ((uint32_t)r >= (uint64_t)msum) continue;
+      const bf16x8 v = *(const bf16x8*)(rows + (int64_t)r * D + c * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)v[e];
+    }
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)acc[e];
+    *(bf16x8*)(out + m * D + c * 8) = o;
+  }
+}
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+inline int check_dims(int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum) {
+  if (M <= 0 || D <= 0 || H <= 0 || N <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
+  if (D % kBK != 0 || H % kBK != 0) return MOMOE_ERR_UNSUPPORTED;
+  if (Msum >= (1ll << 31) || M * D >= (1ll << 40) || D > (1 << 20) || H > (1 << 20))
+    return MOMOE_ERR_UNSUPPORTED;
+  return MOMOE_OK;
+}
+
+inline unsigned grid_for(int64_t Msum, int64_t N, int64_t nb) {
+  const int64_t ub = max_row_tiles(Msum, N, BM) * nb;
+  return (unsigned)(cdiv64(ub, 8) * 8);
+}
+
+}  // namespace
+}  // namespace momoe
+
+using namespace momoe;
+
+extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
+                                     const int32_t* idx_Msum, const int32_t* tile_table,
+                                     void* h_MsumH, void* ab_rows, int64_t ab_row_lo,
+                                     int64_t ab_row_hi, int64_t M, int64_t D, int64_t H,
+                                     int64_t N, int64_t Msum, void* stream) {
+  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || (!h_MsumH && !ab_rows))
+    return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_MsumH & 7) ||
+      ((uintptr_t)ab_rows & 7))
+    return MOMOE_ERR_BAD_ARG;
+  const int st = check_dims(M, D, H, N, Msum);
+  if (st != MOMOE_OK) return st;
+  Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
+             (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H};
+  const unsigned grid = grid_for(Msum, N, cdiv64(H, BN / 2));
+  lin1_swiglu_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  return launch_status();
+}
+
+extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, const float* s_NM,
+                                    int64_t s_stride_n, int64_t s_stride_m,
+                                    const int32_t* idx_Msum, const int32_t* tile_table,
+                                    void* ys_MsumD, int64_t M, int64_t D, int64_t H, int64_t N,
+                                    int64_t Msum, void* stream) {
+  if (!h_MsumH || !Wl2_NHD || !s_NM || !idx_Msum || !tile_table || !ys_MsumD)
+    return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(h_MsumH) || !aligned16(Wl2_NHD) || ((uintptr_t)ys_MsumD & 7))
+    return MOMOE_ERR_BAD_ARG;
+  const int st = check_dims(M, D, H, N, Msum);
+  if (st != MOMOE_OK) return st;
+  Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
+             idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H};
+  const unsigned grid = grid_for(Msum, N, cdiv64(D, BN));
+  lin2_scale_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  return launch_status();
+}
+
+extern "C" int momoe_combine(const void* rows_MsumD, const int32_t* inv_MK, void* out_MD,
+                             int64_t M, int64_t D, int64_t K, int64_t Msum, void* stream) {
+  if (!rows_MsumD || !inv_MK || !out_MD) return MOMOE_ERR_BAD_ARG;
+  if (M <= 0 || D <= 0 || K <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
+  if (D % 8 != 0 || M >= (1ll << 31) || Msum >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  if (!aligned16(rows_MsumD) || !aligned16(out_MD)) return MOMOE_ERR_BAD_ARG;
+  combine_kernel<<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(
+      (const bf16*)rows_MsumD, inv_MK, (bf16*)out_MD, (int)D, (int)K, Msum);
+  return launch_status();
+}

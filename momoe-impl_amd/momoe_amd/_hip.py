@@ -1,0 +1,189 @@
+"""ctypes binding of libmomoe_hip.so (the C ABI declared in include/momoe_hip.h).
+
+The library is the only compute path: if it is missing or fails to load, importing
+this module raises, and every wrapper raises RuntimeError on a non-zero status.
+torch must be imported first so that the HIP runtime already loaded by torch is the
+one the library binds to (both use the SONAME libamdhip64.so.7).
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads the HIP runtime)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmomoe_hip.so")
+
+TILE_ROWS = 128
+GS_BLOCK = 256
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} not found: build it with `python momoe-impl_amd/build.py` "
+        "(there is no fallback compute path)")
+
+_lib = ctypes.CDLL(LIB_PATH)
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+_SIGNATURES = {
+    "momoe_abi_version": (_int, []),
+    "momoe_status_string": (ctypes.c_char_p, [_int]),
+    "momoe_tile_table_ints": (_i64, [_i64, _i64, _i64, _int]),
+    "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
+    "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
+                                 _p, _i64, _p, _p]),
+    "momoe_lin1_swiglu_fwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64,
+                                     _i64, _p]),
+    "momoe_lin2_scale_fwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64,
+                                    _i64, _p]),
+    "momoe_combine": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "momoe_dgrad_h_swiglu_bwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _p, _p, _p,
+                                        _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_gs_scatter": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "momoe_dgrad_x": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "momoe_router_fwd": (_int, [_p, _int, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p]),
+    "momoe_router_bwd": (_int, [_p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+for _name, (_res, _args) in _SIGNATURES.items():
+    _fn = getattr(_lib, _name)  # AttributeError here = library/header mismatch
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+
+def status_string(code):
+    return _lib.momoe_status_string(int(code)).decode()
+
+
+def _check(code, what):
+    if code != 0:
+        raise RuntimeError(f"{what} failed: status {code} ({status_string(code)})")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("momoe_amd kernels need device tensors (no CPU compute path exists)")
+
+
+def abi_version():
+    return _lib.momoe_abi_version()
+
+
+# ---------------------------------------------------------------- index build
+def index_build(mask_NM, K):
+    """mask_NM int32 [N,M] (any strides) -> dict of device tensors.
+    See momoe_index_build in include/momoe_hip.h."""
+    _need_cuda(mask_NM)
+    assert mask_NM.dtype == torch.int32 and mask_NM.dim() == 2
+    N, M = mask_NM.shape
+    dev = mask_NM.device
+    msum = M * K
+    sizes = torch.empty(N, dtype=torch.int64, device=dev)
+    cumsums = torch.empty(N + 1, dtype=torch.int32, device=dev)
+    idx = torch.empty(msum, dtype=torch.int32, device=dev)
+    which = torch.empty(msum, dtype=torch.int32, device=dev)
+    inv = torch.empty(msum, dtype=torch.int32, device=dev)
+    table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, TILE_ROWS), dtype=torch.int32, device=dev)
+    ws_bytes = _lib.momoe_index_workspace_bytes(M, N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    violations = torch.zeros(1, dtype=torch.int32, device=dev)
+    _check(_lib.momoe_index_build(_ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N, K,
+                                  _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv),
+                                  _ptr(table), TILE_ROWS, _ptr(ws), ws_bytes, _ptr(violations),
+                                  _stream()), "momoe_index_build")
+    return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
+            "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
+
+
+# ---------------------------------------------------------------- experts fwd
+def lin1_swiglu_fwd(x_MD, Wl1_ND2H, idx, table, h, ab, ab_lo, ab_hi):
+    _need_cuda(x_MD, Wl1_ND2H)
+    M, D = x_MD.shape
+    N, _, H2 = Wl1_ND2H.shape
+    _check(_lib.momoe_lin1_swiglu_fwd(_ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(h),
+                                      _ptr(ab), ab_lo, ab_hi, M, D, H2 // 2, N, idx.numel(),
+                                      _stream()), "momoe_lin1_swiglu_fwd")
+
+
+def lin2_scale_fwd(h, Wl2_NHD, s_NM, idx, table, ys, M):
+    _need_cuda(h, Wl2_NHD, s_NM)
+    N, H, D = Wl2_NHD.shape
+    _check(_lib.momoe_lin2_scale_fwd(_ptr(h), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
+                                     s_NM.stride(1), _ptr(idx), _ptr(table), _ptr(ys), M, D, H, N,
+                                     idx.numel(), _stream()), "momoe_lin2_scale_fwd")
+
+
+def combine(rows_MsumD, inv_MK, out_MD):
+    M, K = inv_MK.shape
+    D = rows_MsumD.shape[1]
+    _check(_lib.momoe_combine(_ptr(rows_MsumD), _ptr(inv_MK), _ptr(out_MD), M, D, K,
+                              rows_MsumD.shape[0], _stream()), "momoe_combine")
+
+
+# ---------------------------------------------------------------- experts bwd
+def dgrad_h_swiglu_bwd(Gy_MD, Wl2_NHD, s_NM, idx, table, ab_save, Msave, gz, hs, gs_part):
+    M, D = Gy_MD.shape
+    N, H, _ = Wl2_NHD.shape
+    _check(_lib.momoe_dgrad_h_swiglu_bwd(_ptr(Gy_MD), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
+                                         s_NM.stride(1), _ptr(idx), _ptr(table), _ptr(ab_save),
+                                         Msave, _ptr(gz), _ptr(hs), _ptr(gs_part), M, D, H, N,
+                                         idx.numel(), _stream()), "momoe_dgrad_h_swiglu_bwd")
+
+
+def gs_scatter(gs_part, idx, cumsums, Gs_NM):
+    N, M = Gs_NM.shape
+    _check(_lib.momoe_gs_scatter(_ptr(gs_part), gs_part.shape[0], _ptr(idx), _ptr(cumsums),
+                                 _ptr(Gs_NM), M, N, idx.numel(), _stream()), "momoe_gs_scatter")
+
+
+def dgrad_x(gz, Wl1_ND2H, table, gxs, M):
+    N, D, H2 = Wl1_ND2H.shape
+    _check(_lib.momoe_dgrad_x(_ptr(gz), _ptr(Wl1_ND2H), _ptr(table), _ptr(gxs), M, D, H2 // 2, N,
+                              gz.shape[0], _stream()), "momoe_dgrad_x")
+
+
+def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, Msum):
+    N, X, Y = GW_NXY.shape
+    _check(_lib.momoe_wgrad(_ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
+                            B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), N, X, Y,
+                            Msum, _stream()), "momoe_wgrad")
+
+
+# ---------------------------------------------------------------- router
+def router_fwd(logits_MN, biases_N, K, Ks):
+    _need_cuda(logits_MN, biases_N)
+    M, N = logits_MN.shape
+    dev = logits_MN.device
+    assert logits_MN.is_contiguous() and logits_MN.dtype in (torch.bfloat16, torch.float32)
+    mask = torch.empty((N, M), dtype=torch.int32, device=dev)
+    s_MN = torch.empty((M, N), dtype=torch.float32, device=dev)
+    p_sel = torch.empty((M, N), dtype=torch.float32, device=dev)
+    Ng_M = torch.empty(M, dtype=torch.float32, device=dev)
+    Ks_M = torch.empty(M, dtype=torch.float32, device=dev)
+    _check(_lib.momoe_router_fwd(_ptr(logits_MN), int(logits_MN.dtype == torch.float32),
+                                 _ptr(biases_N), M, N, K, Ks, _ptr(mask), _ptr(s_MN), _ptr(p_sel),
+                                 _ptr(Ng_M), _ptr(Ks_M), _stream()), "momoe_router_fwd")
+    return mask, s_MN, p_sel, Ng_M, Ks_M
+
+
+def router_bwd(Gs_NM, p_sel_MN, s_MN, Ng_M, Ks_M, mask_NM, Ks):
+    N, M = Gs_NM.shape
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=Gs_NM.device)
+    _check(_lib.momoe_router_bwd(_ptr(Gs_NM), Gs_NM.stride(0), Gs_NM.stride(1), _ptr(p_sel_MN),
+                                 _ptr(s_MN), _ptr(Ng_M), _ptr(Ks_M), _ptr(mask_NM), M, N, Ks,
+                                 _ptr(out), _stream()), "momoe_router_bwd")
+    return out
