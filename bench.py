@@ -1,0 +1,189 @@
+"""Benchmark of the MoE-layer hot path on one MI355X.
+
+One step = one forward + backward of `MoMoE` (x, mask, s -> y; dy -> dx, dWl1, dWl2, ds)
+on the headline layer: B=4, S=2048 (8192 tokens), D=2048, H=1024, N=128 experts, K=8,
+bf16 with fp32 accumulation, save_percent=0.  Inputs are synthetic, seeded, and resident
+in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "momoe-impl_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None until measured for the kernel that is currently dominant.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def headline_inputs(M, D, H, N, K, seed=0):
+    import torch
+    from helpers import make_routing
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, D, generator=g)
+    dy = torch.randn(M, D, generator=g)
+    W1 = torch.empty(N, D, 2 * H, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
+    W2 = torch.empty(N, H, D, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
+    mask, s = make_routing(M, N, K, 0, seed=seed)
+    return x, W1, W2, mask, s, dy
+
+
+def kernel_flops(D, H, msum):
+    """Algorithmic flops per launch (2*m*n*k per GEMM; recomputation counted separately)."""
+    unit = float(D) * H * msum
+    return {
+        "momoe_lin1_swiglu_fwd": 4 * unit, "momoe_lin2_scale_fwd": 2 * unit,
+        "momoe_dgrad_h_swiglu_bwd": 2 * unit, "momoe_dgrad_x": 4 * unit,
+        "momoe_wgrad[Wl2]": 2 * unit, "momoe_wgrad[Wl1]": 4 * unit,
+    }
+
+
+def cpu_baseline(D, H, N, K, budget_s=20.0):
+    """The oracle MoE layer (router restated in torch + per-expert loop + autograd backward)
+    on the host cores, on a reduced token count of the same layer."""
+    import torch
+    import oracle
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    Ms = 1024
+    x, W1, W2, mask, s, dy = headline_inputs(Ms, D, H, N, K, seed=1)
+    W1f, W2f = W1.float().requires_grad_(), W2.float().requires_grad_()
+    xf = x.bfloat16().float().requires_grad_()
+    sf = s.clone().requires_grad_()
+    times = []
+    t_start = time.time()
+    for it in range(4):
+        t0 = time.time()
+        y = oracle.experts_forward(xf, W1f, W2f, mask, sf)
+        y.backward(dy)
+        dt = time.time() - t0
+        W1f.grad = W2f.grad = xf.grad = sf.grad = None
+        if it > 0:
+            times.append(dt)
+        if time.time() - t_start > budget_s and times:
+            break
+    best = min(times)
+    return {"value": Ms / best, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"oracle MoE layer fwd+bwd, fp32, {Ms} of 8192 tokens of the headline layer "
+                      f"(D={D}, H={H}, N={N}, K={K}), best of {len(times)} runs, {best:.3f} s each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--save-percent", type=float, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import momoe_amd
+    from momoe_amd import _hip
+
+    B, S, D, H, N, K = 4, 2048, 2048, 1024, 128, 8
+    M = B * S
+    msum = M * K
+    dev = "cuda:0"
+    x, W1, W2, mask, s, dy = headline_inputs(M, D, H, N, K)
+    maskd = mask.to(dev)
+    sd = s.T.contiguous().to(dev).T.requires_grad_()
+    xd = x.to(dev, torch.bfloat16).reshape(B, S, D).requires_grad_()
+    dyd = dy.to(dev, torch.bfloat16).reshape(B, S, D)
+
+    def make_layer(sp):
+        return momoe_amd.MoMoE(D, H, N, K, save_percent=sp, Wl1_ND2H=W1.to(dev), Wl2_NHD=W2.to(dev))
+
+    def step(layer):
+        y, _ = layer(xd, maskd, sd)
+        y.backward(dyd)
+        layer.Wl1_ND2H.grad = layer.Wl2_NHD.grad = xd.grad = sd.grad = None
+
+    def timed(layer, fn, steps, warmup):
+        for _ in range(warmup):
+            fn(layer)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn(layer)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def fwd_only(layer):
+        with torch.no_grad():
+            layer(xd, maskd, sd)
+
+    layer = make_layer(args.save_percent)
+    ms = timed(layer, step, args.steps, args.warmup)
+    ms_fwd = timed(layer, fwd_only, args.steps, 2)
+    torch.cuda.reset_peak_memory_stats()
+    base_mem = torch.cuda.memory_allocated()
+    step(layer)
+    torch.cuda.synchronize()
+    peak_extra_mib = (torch.cuda.max_memory_allocated() - base_mem) / 2**20
+
+    # per-kernel launch durations, HIP events on the launch stream, same region
+    per = {}
+    with _hip.kernel_timer() as kt:
+        for _ in range(args.steps):
+            step(layer)
+    wcount = 0
+    for name, t in kt.durations_ms():
+        if name == "momoe_wgrad":
+            name = "momoe_wgrad[Wl2]" if wcount % 2 == 0 else "momoe_wgrad[Wl1]"
+            wcount += 1
+        per.setdefault(name, []).append(t)
+    # lin1 is launched twice per step at save_percent < 100 (forward, backward recomputation)
+    kernels = {k: {"launches_per_step": len(v) / args.steps, "avg_ms": sum(v) / len(v)} for k, v in per.items()}
+    flops = kernel_flops(D, H, msum)
+    for k, f in flops.items():
+        if k in kernels:
+            kernels[k]["tflops"] = f / kernels[k]["avg_ms"] / 1e9
+            kernels[k]["frac_peak"] = kernels[k]["tflops"] / PEAK_BF16_TFLOPS
+    dom = max((k for k in kernels if k in flops),
+              key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS,
+                "avg_launch_ms": kernels[dom]["avg_ms"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom)}
+
+    # the other save setting, and the layer with its router in front
+    other_sp = 100 if args.save_percent == 0 else 0
+    layer2 = make_layer(other_sp)
+    ms_other = timed(layer2, step, max(args.steps // 2, 3), 2)
+    del layer2
+
+    useful = 18.0 * D * H * msum
+    out = {
+        "metric": "moe_layer_fwd_bwd_tokens_per_s", "value": M / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "headline MoE layer fwd+bwd: B=4 S=2048 (8192 tokens) D=2048 H=1024 "
+                               "N=128 K=8, near-uniform top-8 routing of N(0,1) logits",
+                   "save_percent": args.save_percent, "tokens": M, "D": D, "H": H, "experts": N, "top_k": K},
+        "fwd_bwd_tflops": useful / ms / 1e9, "fwd_bwd_frac_bf16_peak": useful / ms / 1e9 / PEAK_BF16_TFLOPS,
+        "fwd_ms": ms_fwd, "fwd_tokens_per_s": M / (ms_fwd * 1e-3),
+        "fwd_tflops": 6.0 * D * H * msum / ms_fwd / 1e9,
+        f"ms_per_step_save_percent_{other_sp}": ms_other,
+        "peak_activation_mib": peak_extra_mib,
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(D, H, N, K)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,152 @@
+// Weight-gradient grouped GEMM: GW[i] = A_i^T . B_i, contracting over the sorted
+// rows of expert i.  Both operands are stored [row][feature], i.e. k-strided, so
+// both go through the LDS transpose read.  Rows may be gathered through an index
+// (x and G_y are never materialised in sorted order).
+#include "gemm_tile.hpp"
+
+namespace momoe {
+namespace {
+
+constexpr int BX = 128;  // output rows per tile (features of A)
+constexpr int BY = 256;  // output columns per tile (features of B)
+constexpr int FM = 2, FN = 4;
+
+// k-strided operand whose k-rows are the rows [row_begin,row_end) of an expert,
+// optionally gathered; rows past row_end are zero-filled.
+template <int COLS>
+struct TGatherOperand {
+  static constexpr int LD = COLS + 16;
+  static constexpr int CPR = COLS / 8;
+  static constexpr int KSTEP = kThreads / CPR;
+  static constexpr int NCH = kBK / KSTEP;
+  static constexpr int LDS_ELEMS = kBK * LD;
+  const bf16* base;  // column offset applied; nullptr when this thread's 8 columns are out of range
+  int64_t ld;
+  const int32_t* gather;
+  int row_begin, row_end;
+  int32_t rowid[NCH];
+  u32x4 stage[NCH];
+
+  __device__ __forceinline__ void fetch_rows(int kt) {
+    const int kr = threadIdx.x / CPR;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int rr = row_begin + kt * kBK + kr + j * KSTEP;
+      int32_t id = -1;
+      if (rr < row_end) id = gather ? gather[rr] : rr;
+      rowid[j] = id;
+    }
+  }
+  __device__ __forceinline__ void init(const bf16* mat, int64_t ld_, const int32_t* gather_,
+                                       int col0, int ncols, int rb, int re) {
+    const int cc = threadIdx.x % CPR;
+    const int c = col0 + cc * 8;
+    base = c < ncols ? mat + c : nullptr;
+    ld = ld_;
+    gather = gather_;
+    row_begin = rb;
+    row_end = re;
+    fetch_rows(0);
+  }
+  // uses the row ids fetched for stage kt, then fetches those of stage kt+1
+  __device__ __forceinline__ void load(int kt) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      if (base != nullptr && rowid[j] >= 0) stage[j] = *(const u32x4*)(base + (int64_t)rowid[j] * ld);
+      else stage[j] = u32x4{0, 0, 0, 0};
+    }
+    fetch_rows(kt + 1);
+  }
+  __device__ __forceinline__ void store(bf16* lds) const {
+    const int cc = threadIdx.x % CPR, kr = threadIdx.x / CPR;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) *(u32x4*)(lds + (kr + j * KSTEP) * LD + cc * 8) = stage[j];
+  }
+  static __device__ __forceinline__ bf16x8 frag(const bf16* lds, int c0, int kk) {
+    return TOperand<COLS>::frag(lds, c0, kk);
+  }
+};
+
+struct WgradArgs {
+  const bf16* a;
+  int64_t lda;
+  const int32_t* ga;
+  const bf16* b;
+  int64_t ldb;
+  const int32_t* gb;
+  const int32_t* cumsums;
+  bf16* gw;
+  int N, X, Y;
+  int tiles_x, tiles_y;
+};
+
+// 1-D grid.  id%8 is the XCD a workgroup lands on; experts are dealt round-robin to the
+// XCDs and every tile of an expert runs on that one XCD, so the expert's rows are
+// fetched from HBM once and re-read from that XCD's L2.
+__global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
+  using AOp = TGatherOperand<BX>;
+  using BOp = TGatherOperand<BY>;
+  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  const int tpe = p.tiles_x * p.tiles_y;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int expert = (slot / tpe) * 8 + xcd;
+  if (expert >= p.N) return;
+  const int q = slot % tpe;
+  const int tx = q / p.tiles_y, ty = q % p.tiles_y;
+  const int rb = p.cumsums[expert], re = p.cumsums[expert + 1];
+  const int x0 = tx * BX, y0 = ty * BY;
+
+  AOp A;
+  BOp B;
+  A.init(p.a, p.lda, p.ga, x0, p.X, rb, re);
+  B.init(p.b, p.ldb, p.gb, y0, p.Y, rb, re);
+
+  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
+  const int m_org[FM] = {wm * 64, wm * 64 + 32};
+  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
+  f32x16 acc[FN][FM];
+  zero_acc<FM, FN>(acc);
+  const int ktiles = (re - rb + kBK - 1) / kBK;
+  if (ktiles > 0) gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, ktiles, lds, m_org, n_org);
+
+  bf16* out = p.gw + (int64_t)expert * p.X * p.Y;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int x = x0 + m_org[i] + acc_row();
+    if (x >= p.X) continue;
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int y = y0 + n_org[f] + acc_col(qd);
+        if (y >= p.Y) continue;
+        store_bf16x4(out + (int64_t)x * p.Y + y, acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
+                     acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]);
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace momoe
+
+using namespace momoe;
+
+extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
+                           const void* B_rows, int64_t ldb, const int32_t* b_gather,
+                           const int32_t* cumsums_N1, void* GW_NXY, int64_t N, int64_t X,
+                           int64_t Y, int64_t Msum, void* stream) {
+  if (!A_rows || !B_rows || !cumsums_N1 || !GW_NXY) return MOMOE_ERR_BAD_ARG;
+  if (N <= 0 || X <= 0 || Y <= 0 || Msum <= 0 || lda < X || ldb < Y) return MOMOE_ERR_BAD_ARG;
+  if (X % 8 != 0 || Y % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return MOMOE_ERR_UNSUPPORTED;
+  if (((uintptr_t)A_rows & 15) || ((uintptr_t)B_rows & 15) || ((uintptr_t)GW_NXY & 7))
+    return MOMOE_ERR_BAD_ARG;
+  if (Msum >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
+  const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
+  const int64_t blocks = cdiv64(N, 8) * 8 * tiles_x * tiles_y;
+  if (blocks >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
+              (bf16*)GW_NXY, (int)N, (int)X, (int)Y, tiles_x, tiles_y};
+  wgrad_kernel<<<(unsigned)blocks, kThreads, 0, (hipStream_t)stream>>>(a);
+  return launch_status();
+}

@@ -60,9 +60,42 @@ def status_string(code):
     return _lib.momoe_status_string(int(code)).decode()
 
 
-def _check(code, what):
+_TIMINGS = None  # list of (entry point, start event, end event) while kernel_timer() is active
+
+
+class kernel_timer:
+    """Context manager: record a HIP event pair around every C-ABI call made inside it
+    (on torch's current stream).  `durations_ms()` synchronises and returns
+    [(entry point, milliseconds), ...] in call order."""
+
+    def __enter__(self):
+        global _TIMINGS
+        self.records = _TIMINGS = []
+        return self
+
+    def __exit__(self, *exc):
+        global _TIMINGS
+        _TIMINGS = None
+        return False
+
+    def durations_ms(self):
+        torch.cuda.synchronize()
+        return [(name, a.elapsed_time(b)) for name, a, b in self.records]
+
+
+def _call(name, *args):
+    fn = getattr(_lib, name)
+    if _TIMINGS is None:
+        code = fn(*args)
+    else:
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        code = fn(*args)
+        b.record()
+        _TIMINGS.append((name, a, b))
     if code != 0:
-        raise RuntimeError(f"{what} failed: status {code} ({status_string(code)})")
+        raise RuntimeError(f"{name} failed: status {code} ({status_string(code)})")
 
 
 def _ptr(t):
@@ -101,10 +134,10 @@ def index_build(mask_NM, K):
     ws_bytes = _lib.momoe_index_workspace_bytes(M, N)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     violations = torch.zeros(1, dtype=torch.int32, device=dev)
-    _check(_lib.momoe_index_build(_ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N, K,
+    _call("momoe_index_build", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N, K,
                                   _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv),
                                   _ptr(table), TILE_ROWS, _ptr(ws), ws_bytes, _ptr(violations),
-                                  _stream()), "momoe_index_build")
+                                  _stream())
     return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
             "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
 
@@ -114,53 +147,53 @@ def lin1_swiglu_fwd(x_MD, Wl1_ND2H, idx, table, h, ab, ab_lo, ab_hi):
     _need_cuda(x_MD, Wl1_ND2H)
     M, D = x_MD.shape
     N, _, H2 = Wl1_ND2H.shape
-    _check(_lib.momoe_lin1_swiglu_fwd(_ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(h),
+    _call("momoe_lin1_swiglu_fwd", _ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(h),
                                       _ptr(ab), ab_lo, ab_hi, M, D, H2 // 2, N, idx.numel(),
-                                      _stream()), "momoe_lin1_swiglu_fwd")
+                                      _stream())
 
 
 def lin2_scale_fwd(h, Wl2_NHD, s_NM, idx, table, ys, M):
     _need_cuda(h, Wl2_NHD, s_NM)
     N, H, D = Wl2_NHD.shape
-    _check(_lib.momoe_lin2_scale_fwd(_ptr(h), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
+    _call("momoe_lin2_scale_fwd", _ptr(h), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
                                      s_NM.stride(1), _ptr(idx), _ptr(table), _ptr(ys), M, D, H, N,
-                                     idx.numel(), _stream()), "momoe_lin2_scale_fwd")
+                                     idx.numel(), _stream())
 
 
 def combine(rows_MsumD, inv_MK, out_MD):
     M, K = inv_MK.shape
     D = rows_MsumD.shape[1]
-    _check(_lib.momoe_combine(_ptr(rows_MsumD), _ptr(inv_MK), _ptr(out_MD), M, D, K,
-                              rows_MsumD.shape[0], _stream()), "momoe_combine")
+    _call("momoe_combine", _ptr(rows_MsumD), _ptr(inv_MK), _ptr(out_MD), M, D, K,
+                              rows_MsumD.shape[0], _stream())
 
 
 # ---------------------------------------------------------------- experts bwd
 def dgrad_h_swiglu_bwd(Gy_MD, Wl2_NHD, s_NM, idx, table, ab_save, Msave, gz, hs, gs_part):
     M, D = Gy_MD.shape
     N, H, _ = Wl2_NHD.shape
-    _check(_lib.momoe_dgrad_h_swiglu_bwd(_ptr(Gy_MD), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
+    _call("momoe_dgrad_h_swiglu_bwd", _ptr(Gy_MD), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
                                          s_NM.stride(1), _ptr(idx), _ptr(table), _ptr(ab_save),
                                          Msave, _ptr(gz), _ptr(hs), _ptr(gs_part), M, D, H, N,
-                                         idx.numel(), _stream()), "momoe_dgrad_h_swiglu_bwd")
+                                         idx.numel(), _stream())
 
 
 def gs_scatter(gs_part, idx, cumsums, Gs_NM):
     N, M = Gs_NM.shape
-    _check(_lib.momoe_gs_scatter(_ptr(gs_part), gs_part.shape[0], _ptr(idx), _ptr(cumsums),
-                                 _ptr(Gs_NM), M, N, idx.numel(), _stream()), "momoe_gs_scatter")
+    _call("momoe_gs_scatter", _ptr(gs_part), gs_part.shape[0], _ptr(idx), _ptr(cumsums),
+                                 _ptr(Gs_NM), M, N, idx.numel(), _stream())
 
 
 def dgrad_x(gz, Wl1_ND2H, table, gxs, M):
     N, D, H2 = Wl1_ND2H.shape
-    _check(_lib.momoe_dgrad_x(_ptr(gz), _ptr(Wl1_ND2H), _ptr(table), _ptr(gxs), M, D, H2 // 2, N,
-                              gz.shape[0], _stream()), "momoe_dgrad_x")
+    _call("momoe_dgrad_x", _ptr(gz), _ptr(Wl1_ND2H), _ptr(table), _ptr(gxs), M, D, H2 // 2, N,
+                              gz.shape[0], _stream())
 
 
 def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, Msum):
     N, X, Y = GW_NXY.shape
-    _check(_lib.momoe_wgrad(_ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
+    _call("momoe_wgrad", _ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
                             B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), N, X, Y,
-                            Msum, _stream()), "momoe_wgrad")
+                            Msum, _stream())
 
 
 # ---------------------------------------------------------------- router
@@ -174,16 +207,16 @@ def router_fwd(logits_MN, biases_N, K, Ks):
     p_sel = torch.empty((M, N), dtype=torch.float32, device=dev)
     Ng_M = torch.empty(M, dtype=torch.float32, device=dev)
     Ks_M = torch.empty(M, dtype=torch.float32, device=dev)
-    _check(_lib.momoe_router_fwd(_ptr(logits_MN), int(logits_MN.dtype == torch.float32),
+    _call("momoe_router_fwd", _ptr(logits_MN), int(logits_MN.dtype == torch.float32),
                                  _ptr(biases_N), M, N, K, Ks, _ptr(mask), _ptr(s_MN), _ptr(p_sel),
-                                 _ptr(Ng_M), _ptr(Ks_M), _stream()), "momoe_router_fwd")
+                                 _ptr(Ng_M), _ptr(Ks_M), _stream())
     return mask, s_MN, p_sel, Ng_M, Ks_M
 
 
 def router_bwd(Gs_NM, p_sel_MN, s_MN, Ng_M, Ks_M, mask_NM, Ks):
     N, M = Gs_NM.shape
     out = torch.empty((M, N), dtype=torch.bfloat16, device=Gs_NM.device)
-    _check(_lib.momoe_router_bwd(_ptr(Gs_NM), Gs_NM.stride(0), Gs_NM.stride(1), _ptr(p_sel_MN),
+    _call("momoe_router_bwd", _ptr(Gs_NM), Gs_NM.stride(0), Gs_NM.stride(1), _ptr(p_sel_MN),
                                  _ptr(s_MN), _ptr(Ng_M), _ptr(Ks_M), _ptr(mask_NM), M, N, Ks,
-                                 _ptr(out), _stream()), "momoe_router_bwd")
+                                 _ptr(out), _stream())
     return out

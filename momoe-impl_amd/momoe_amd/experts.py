@@ -1,0 +1,176 @@
+"""`MoMoE`: the experts of a SwiGLU mixture-of-experts layer, forward and backward,
+on the gfx950 kernels of libmomoe_hip.so.
+
+Mirrors the module and autograd contract of the reference (momoe/momoe.py:847-972):
+`MoMoE(embedding_dim, intermediate_dim, num_experts, num_chosen_experts, save_percent,
+Wl1_ND2H, Wl2_NHD)`, `forward(x_BSD, mask_NM, s_NM) -> (y_BSD bf16, sizes_N int64)`;
+gradients for x (bf16), Wl1/Wl2 (bf16) and s_NM (fp32 [N,M], zero off-mask).
+
+All temporaries are torch allocations made here; the library never allocates.
+Nothing in this file synchronises with the device: every launch is sized from
+static upper bounds and the routing-dependent tile list lives in device memory.
+"""
+import torch
+import torch.nn as nn
+
+from . import _hip
+
+
+def _saved_rows(msum, save_percent):
+    # momoe/momoe.py:251
+    return int(msum * save_percent / 100.0)
+
+
+class MoEFunction(torch.autograd.Function):
+    """(x_BSD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, K, save_percent) -> (y_BSD, sizes_N).
+
+    Forward (momoe/momoe.py:856-874): routing index, x.Wl1 with fused SwiGLU,
+    h.Wl2 scaled by the gate weight, K-way combine.  With save_percent > 0 the
+    pre-activation halves a|b of the first `Msave` sorted rows are kept for the
+    backward; everything else is recomputed there.
+
+    Backward (momoe/momoe.py:881-903).  Differences from the reference that do not
+    change results beyond rounding: x and G_y are gathered inside the GEMM loads
+    instead of being materialised in sorted order; dL/ds is obtained from
+    (G_y.Wl2^T).h, which equals G_y.(h.Wl2), so the down projection is never
+    recomputed and y_pre is never saved; dL/ds is reduced without atomics.
+    """
+
+    @staticmethod
+    def forward(ctx, x_BSD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, K, save_percent):
+        B, S, D = x_BSD.shape
+        dev = Wl1_ND2H.device
+        assert Wl1_ND2H.device == Wl2_NHD.device, (
+            "All weights must be on the same device, but got: Wl1_ND2H.device = {}, "
+            "Wl2_NHD.device = {}".format(Wl1_ND2H.device, Wl2_NHD.device))
+        if dev.type != "cuda":
+            raise RuntimeError("MoMoE weights must live on the GPU: there is no CPU compute path")
+        N, Dw, H2 = Wl1_ND2H.shape
+        H = H2 // 2
+        assert Dw == D and tuple(Wl2_NHD.shape) == (N, H, D)
+        M = B * S
+
+        with torch.cuda.device(dev):
+            x_MD = x_BSD.reshape(M, D).to(device=dev, dtype=torch.bfloat16).contiguous()
+            W1 = Wl1_ND2H.to(torch.bfloat16).contiguous()
+            W2 = Wl2_NHD.to(torch.bfloat16).contiguous()
+            mask = mask_NM.to(device=dev, dtype=torch.int32)
+            s = s_NM.to(device=dev, dtype=torch.float32)
+
+            ib = _hip.index_build(mask, K)
+            idx, table = ib["idx_Msum"], ib["tile_table"]
+            msum = M * K
+            msave = _saved_rows(msum, save_percent)
+
+            h = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
+            ab_save = torch.empty((msave, 2 * H), device=dev, dtype=torch.bfloat16) if msave > 0 else None
+            _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, h, ab_save, 0, msave)
+            ys = torch.empty((msum, D), device=dev, dtype=torch.bfloat16)
+            _hip.lin2_scale_fwd(h, W2, s, idx, table, ys, M)
+            del h
+            y_MD = torch.empty((M, D), device=dev, dtype=torch.bfloat16)
+            _hip.combine(ys, ib["inv_MK"], y_MD)
+            del ys
+
+        ctx.K = K
+        ctx.msave = msave
+        ctx.has_save = ab_save is not None
+        saved = [x_MD, s, idx, ib["inv_MK"], ib["cumsums_N"], table, W1, W2]
+        if ab_save is not None:
+            saved.append(ab_save)
+        ctx.save_for_backward(*saved)
+        ctx.routing_violations = ib["violations"]
+        sizes_N = ib["sizes_N"]
+        ctx.mark_non_differentiable(sizes_N)
+        return y_MD.view(B, S, D).to(device=x_BSD.device), sizes_N
+
+    @staticmethod
+    def backward(ctx, G_y_BSD, _):
+        saved = ctx.saved_tensors
+        x_MD, s, idx, inv, cumsums, table, W1, W2 = saved[:8]
+        ab_save = saved[8] if ctx.has_save else None
+        msave = ctx.msave
+        B, S, D = G_y_BSD.shape
+        M = B * S
+        N, H, _ = W2.shape
+        msum = idx.numel()
+        dev = W1.device
+        need_x, need_w1, need_w2, _, need_s = ctx.needs_input_grad[:5]
+
+        with torch.cuda.device(dev):
+            Gy = G_y_BSD.reshape(M, D).to(device=dev, dtype=torch.bfloat16).contiguous()
+
+            # a|b for the rows that were not saved are recomputed straight into the buffer
+            # that the next kernel turns, in place, into [G_a|G_b].
+            gz = torch.empty((msum, 2 * H), device=dev, dtype=torch.bfloat16)
+            if msave < msum:
+                _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, None, gz, msave, msum)
+            hs = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
+            nparts = (H + _hip.GS_BLOCK - 1) // _hip.GS_BLOCK
+            gs_part = torch.empty((nparts, msum), device=dev, dtype=torch.float32)
+            _hip.dgrad_h_swiglu_bwd(Gy, W2, s, idx, table, ab_save, msave, gz, hs, gs_part)
+
+            G_s = None
+            if need_s:
+                G_s = torch.zeros((N, M), device=dev, dtype=torch.float32)
+                _hip.gs_scatter(gs_part, idx, cumsums, G_s)
+            del gs_part
+
+            G_W2 = None
+            if need_w2:
+                G_W2 = torch.empty_like(W2)
+                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, msum)
+            del hs
+
+            G_W1 = None
+            if need_w1:
+                G_W1 = torch.empty_like(W1)
+                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, msum)
+
+            G_x_BSD = None
+            if need_x:
+                gxs = torch.empty((msum, D), device=dev, dtype=torch.bfloat16)
+                _hip.dgrad_x(gz, W1, table, gxs, M)
+                G_x = torch.empty((M, D), device=dev, dtype=torch.bfloat16)
+                _hip.combine(gxs, inv, G_x)
+                del gxs
+                G_x_BSD = G_x.view(B, S, D).to(G_y_BSD.device)
+        return G_x_BSD, G_W1, G_W2, None, G_s, None, None
+
+
+class MoMoE(nn.Module):
+    """Memory-optimised mixture of SwiGLU experts (momoe/momoe.py:914-972).
+
+    Args:
+        embedding_dim: D.  intermediate_dim: H.  num_experts: N (shared experts included,
+        as the last rows of mask_NM/s_NM).  num_chosen_experts: K per token (shared included).
+        save_percent: share of the (token, expert) rows whose pre-activations are kept
+        for the backward, 0..100.
+        Wl1_ND2H / Wl2_NHD: optional initial weights, [N, D, 2H] and [N, H, D]; the first
+        H columns of Wl1 are the linear half, the last H go through SiLU.
+    D and H must be multiples of 32.
+    """
+
+    def __init__(self, embedding_dim, intermediate_dim, num_experts, num_chosen_experts,
+                 save_percent=0, Wl1_ND2H=None, Wl2_NHD=None):
+        assert save_percent >= 0 and save_percent <= 100, (
+            "save_percent must be between 0 and 100 inclusive, got {}".format(save_percent))
+        super().__init__()
+        self.D = embedding_dim
+        self.H = intermediate_dim
+        self.N = num_experts
+        self.K = num_chosen_experts
+        self.save_percent = save_percent
+
+        if Wl1_ND2H is None:
+            Wl1_ND2H = torch.randn((self.N, self.D, 2 * self.H), device="cuda", dtype=torch.bfloat16) / self.D
+        if Wl2_NHD is None:
+            Wl2_NHD = torch.randn((self.N, self.H, self.D), device="cuda", dtype=torch.bfloat16) / self.D
+        self.Wl1_ND2H = nn.Parameter(Wl1_ND2H.clone().detach().to(torch.bfloat16), requires_grad=True)
+        self.Wl2_NHD = nn.Parameter(Wl2_NHD.clone().detach().to(torch.bfloat16), requires_grad=True)
+
+    def forward(self, x_BSD, mask_NM, s_NM):
+        """x_BSD [B,S,D]; mask_NM int32 0/1 [N,M] with exactly K ones per token; s_NM [N,M]
+        gate weights (zero off-mask).  Returns (y_BSD bf16, tokens per expert int64 [N])."""
+        return MoEFunction.apply(x_BSD, self.Wl1_ND2H, self.Wl2_NHD, mask_NM, s_NM, self.K,
+                                 self.save_percent)

@@ -1,0 +1,75 @@
+"""GPU: routing index build through the C ABI, bit-exact against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import make_routing
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(mask, K):
+    from momoe_amd import _hip
+    out = _hip.index_build(mask.to("cuda:0"), K)
+    torch.cuda.synchronize()
+    return {k: v.cpu() for k, v in out.items()}
+
+
+def _compare(mask, K, out):
+    o = oracle.index_build(mask)
+    assert out["sizes_N"].dtype == torch.int64 and out["cumsums_N"].dtype == torch.int32
+    for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum"):
+        assert np.array_equal(out[k].numpy(), o[k]), k
+    assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
+    assert out["violations"].item() == 0
+    # tile table: every expert's rows are covered exactly once, in order
+    t = out["tile_table"].numpy()
+    nt, bm = int(t[0]), int(t[1])
+    ent = t[4:4 + 4 * nt].reshape(nt, 4)
+    expect = []
+    for i, (c0, sz) in enumerate(zip(o["cumsums_N"][:-1], o["sizes_N"])):
+        first = len(expect)
+        for _ in range(-(-int(sz) // bm)):
+            expect.append((i, first, int(c0), int(sz)))
+    assert ent.tolist() == [list(e) for e in expect]
+
+
+@pytest.mark.parametrize("M,N,K,Ks,skew", [
+    (128, 8, 2, 0, None),       # the tiny CPU-reference configuration
+    (8192, 128, 8, 0, None),    # headline routing
+    (1000, 60, 6, 0, None),     # M not a multiple of the 256-token panel, N not of the 16-expert panel
+    (16384, 64, 8, 4, 1.8),     # skewed routing + 4 shared experts (full rows)
+    (16, 128, 8, 0, None),      # decode-sized
+    (1, 4, 4, 0, None),
+    (65536, 64, 8, 0, None),    # largest token count of the configurations
+])
+def test_index_bit_exact(M, N, K, Ks, skew):
+    mask, _ = make_routing(M, N, K, Ks, seed=11, skew=skew)
+    _compare(mask, K, _run(mask, K))
+
+
+def test_index_strided_mask():
+    mask, _ = make_routing(777, 24, 3, seed=2)
+    strided = mask.T.contiguous().to("cuda:0").T  # strides (1, N)
+    from momoe_amd import _hip
+    out = {k: v.cpu() for k, v in _hip.index_build(strided, 3).items()}
+    _compare(mask, 3, out)
+
+
+def test_violation_counter_and_no_out_of_bounds():
+    mask, _ = make_routing(512, 16, 4, seed=3)
+    bad = mask.clone()
+    bad[:, 5] = 0          # token 5 has no expert
+    bad[0:6, 9] = 1        # token 9 has more than K
+    out = _run(bad, 4)
+    assert out["violations"].item() >= 2
+
+
+def test_experts_without_tokens():
+    mask = torch.zeros(8, 300, dtype=torch.int32)
+    mask[1] = 1
+    mask[6] = 1
+    out = _run(mask, 2)
+    _compare(mask, 2, out)
+    assert out["sizes_N"].tolist() == [0, 300, 0, 0, 0, 0, 300, 0]

@@ -1,0 +1,118 @@
+"""GPU: TopKRouter kernels and the MoE wrapper against the oracle."""
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _logits(M, N, seed):
+    return torch.randn(M, N, generator=torch.Generator().manual_seed(seed))
+
+
+@pytest.mark.parametrize("M,N,K,Ks,f32", [
+    (128, 8, 2, 0, True), (8192, 128, 8, 0, True), (1000, 64, 8, 4, True),
+    (513, 200, 6, 1, True), (2048, 128, 8, 0, False),
+])
+def test_router_forward(M, N, K, Ks, f32):
+    from momoe_amd import _hip
+    lg = _logits(M, N, 1)
+    if not f32:
+        lg = lg.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(2)
+    bias = torch.cat([torch.randn(N - Ks, generator=g) * 1e-3, torch.full((Ks,), float("-inf"))])
+    ref = oracle.router_forward(None, None, bias, N, K, Ks, logits=lg.float())
+    mask, s_MN, p_sel, Ng_M, Ks_M = _hip.router_fwd(lg.to("cuda:0"), bias.to("cuda:0"), K, Ks)
+    torch.cuda.synchronize()
+    if f32:
+        assert torch.equal(mask.cpu(), ref["mask_NM"])  # routing bit-exact on tie-free fp32 logits
+    else:
+        # bf16 logits contain exact ties, whose order torch.topk leaves unspecified:
+        # compare only tokens whose K-th and (K+1)-th scores differ
+        sc = torch.softmax(lg.float()[:, :N - Ks], -1) + bias[:N - Ks]
+        top = torch.topk(sc, K - Ks + 1, dim=-1).values
+        clear = (top[:, -2] - top[:, -1]) > 1e-6
+        assert clear.float().mean() > 0.9
+        assert torch.equal(mask.cpu()[:, clear], ref["mask_NM"][:, clear])
+        return
+    assert mask.dtype == torch.int32 and mask.is_contiguous()
+    torch.testing.assert_close(s_MN.cpu(), ref["s_NM"].T, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(p_sel.cpu(), ref["p_sel_MN"], rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(Ng_M.cpu(), ref["Ng_M"], rtol=1e-5, atol=1e-7)
+    if Ks:
+        torch.testing.assert_close(Ks_M.cpu(), ref["Ks_M"], rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("M,N,K,Ks", [(256, 16, 4, 0), (1000, 64, 8, 4), (300, 130, 5, 2)])
+def test_router_backward(M, N, K, Ks):
+    from momoe_amd import _hip
+    lg = _logits(M, N, 3)
+    bias = torch.cat([torch.zeros(N - Ks), torch.full((Ks,), float("-inf"))])
+    ref = oracle.router_forward(None, None, bias, N, K, Ks, logits=lg)
+    G_s = torch.randn(N, M, generator=torch.Generator().manual_seed(4)) * (ref["mask_NM"] != 0)
+    want = oracle.router_backward_closed_form(G_s, ref["p_sel_MN"], ref["s_NM"], ref["Ng_M"], ref["Ks_M"],
+                                              ref["mask_NM"], Ks, round_bf16=True)
+    d = lambda t: t.contiguous().to("cuda:0")
+    got = _hip.router_bwd(d(G_s), d(ref["p_sel_MN"]), d(ref["s_NM"].T), d(ref["Ng_M"]), d(ref["Ks_M"]),
+                          d(ref["mask_NM"]), Ks)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-6)
+    # strided G_s (transposed view) gives the same answer
+    got2 = _hip.router_bwd(d(G_s.T).T, d(ref["p_sel_MN"]), d(ref["s_NM"].T), d(ref["Ng_M"]),
+                           d(ref["Ks_M"]), d(ref["mask_NM"]), Ks)
+    assert torch.equal(got, got2)
+
+
+def test_moe_wrapper_against_oracle_and_state_dict():
+    import momoe_amd
+    torch.manual_seed(0)
+    B, S, D, H, N, K, Ks = 2, 256, 256, 128, 16, 4, 1
+    Wg = torch.randn(D, N) * 0.1
+    W1 = torch.randn(N, D, 2 * H) * 0.02
+    W2 = torch.randn(N, H, D) * 0.02
+    x = torch.randn(B, S, D)
+    dy = torch.randn(B, S, D)
+    moe = momoe_amd.MoE(D, H, N, K, Ks, save_percent=0, bias_update_rate=1e-2,
+                        Wg_DN=Wg.cuda(), Wl1_ND2H=W1.cuda(), Wl2_NHD=W2.cuda())
+    assert set(moe.state_dict().keys()) == {"biases_N", "router.Wg_DN", "momoe.Wl1_ND2H", "momoe.Wl2_NHD"}
+    ref = oracle.OracleMoE(D, H, N, K, Ks, bias_update_rate=1e-2, Wg_DN=Wg, Wl1_ND2H=W1.bfloat16(),
+                           Wl2_NHD=W2.bfloat16())
+    ref.load_state_dict({k: v.cpu().float() if "Wl" in k else v.cpu() for k, v in moe.state_dict().items()})
+    xd = x.cuda().bfloat16().requires_grad_()
+    xo = x.bfloat16().float().requires_grad_()
+    y = moe(xd)
+    yo = ref(xo)
+    y.backward(dy.cuda().bfloat16())
+    yo.backward(dy.bfloat16().float())
+    torch.cuda.synchronize()
+    from gpu_util import assert_close
+    # routing decisions must agree for the comparison to be meaningful (bf16 gate logits can tie)
+    assert torch.equal(moe.biases_N.cpu(), ref.biases_N)
+    assert_close(y, yo, "MoE y")
+    assert_close(xd.grad, xo.grad, "MoE G_x", rel=2e-2)
+    assert_close(moe.router.Wg_DN.grad, ref.router.Wg_DN.grad, "G_Wg", rel=3e-2)
+    assert_close(moe.momoe.Wl2_NHD.grad, ref.momoe.Wl2_NHD.grad, "G_W2", rel=2e-2)
+    assert moe.biases_N[-1].item() == float("-inf")
+
+
+def test_training_smoke_loss_decreases():
+    # scaled-down version of the reference's only test (momoe/test.py): AdamW on
+    # mean((y - x)^2); the loss starts near 1 and must go down.
+    import momoe_amd
+    torch.manual_seed(0)
+    B, S, D, H, N, K, Ks = 4, 1024, 256, 128, 32, 6, 1
+    x = torch.randn(B, S, D, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    moe = momoe_amd.MoE(D, H, N, K, Ks, save_percent=0, bias_update_rate=1e-4)
+    opt = torch.optim.AdamW(moe.parameters(), lr=1e-3)
+    losses = []
+    for _ in range(40):
+        y = moe(x)
+        loss = torch.mean(torch.square(y.float() - x.float()))
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        losses.append(loss.item())
+    assert 0.5 < losses[0] < 1.5
+    assert losses[-1] < 0.9 * losses[0]
