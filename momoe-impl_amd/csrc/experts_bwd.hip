@@ -10,6 +10,9 @@ constexpr int BM = MOMOE_TILE_ROWS;
 constexpr int BN = 256;
 constexpr int FM = 2, FN = 4;
 static_assert(BN == MOMOE_GS_BLOCK, "gs_part blocks follow the column tile");
+using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
+using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
+constexpr size_t kBwdLds = gemm_lds_bytes<RowsA, RowsB>();
 
 struct DhArgs {
   const bf16* gy;
@@ -29,9 +32,9 @@ struct DhArgs {
 
 // u = G_y[idx] . Wl2^T is an "NT" GEMM: both operands are k-contiguous (k = D).
 __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
-  using AOp = ROperand<BM>;
-  using BOp = ROperand<BN>;
-  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  using AOp = RowsA;
+  using BOp = RowsB;
+  bf16* lds = dyn_lds();
   const int D = p.D, H = p.H;
   const int nb = (H + BN - 1) / BN;
   const TileCoord tc = decode_tile(p.table, nb);
@@ -51,7 +54,8 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
   zero_acc<FM, FN>(acc);
   gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, D / kBK, lds, m_org, n_org);
 
-  float* red = (float*)lds;  // [2][BM], LDS stages are free after the main loop's last barrier
+  __syncthreads();           // every wave is done with the LDS stages
+  float* red = (float*)lds;  // [2][BM]
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int rloc = m_org[i] + acc_row();
@@ -108,9 +112,9 @@ struct DxArgs {
 
 // gxs = gz . Wl1^T: contraction over the 2H contiguous columns of both operands.
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
-  using AOp = ROperand<BM>;
-  using BOp = ROperand<BN>;
-  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  using AOp = RowsA;
+  using BOp = RowsB;
+  bf16* lds = dyn_lds();
   const int D = p.D, H2 = 2 * p.H;
   const int nb = (D + BN - 1) / BN;
   const TileCoord tc = decode_tile(p.table, nb);
@@ -205,7 +209,9 @@ extern "C" int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD, 
            tile_table, (const bf16*)ab_save, Msave, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part,
            Msum, (int)D, (int)H};
   const unsigned grid = grid_for(Msum, N, cdiv64(H, BN));
-  dgrad_h_swiglu_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  static std::once_flag once;
+  allow_lds(dgrad_h_swiglu_kernel, kBwdLds, once);
+  dgrad_h_swiglu_kernel<<<grid, kThreads, kBwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -231,6 +237,8 @@ extern "C" int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H,
   DxArgs a{(const bf16*)gz_Msum2H, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
            (int)H};
   const unsigned grid = grid_for(Msum, N, cdiv64(D, BN));
-  dgrad_x_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  static std::once_flag once;
+  allow_lds(dgrad_x_kernel, kBwdLds, once);
+  dgrad_x_kernel<<<grid, kThreads, kBwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }

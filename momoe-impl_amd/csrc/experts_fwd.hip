@@ -8,6 +8,9 @@ namespace {
 constexpr int BM = MOMOE_TILE_ROWS;  // 128 sorted rows per tile
 constexpr int BN = 256;              // output columns per tile
 constexpr int FM = 2, FN = 4;        // 2x2 waves, each 64 rows x 128 columns
+using Lin1A = RDma<BM>;              // token rows, k-contiguous
+using Lin1B = TDma<BN>;              // expert weights [k][col], k-strided
+constexpr size_t kFwdLds = gemm_lds_bytes<Lin1A, Lin1B>();
 
 struct Lin1Args {
   const bf16* x;
@@ -23,9 +26,9 @@ struct Lin1Args {
 // Tile = 128 rows x (128 `a` columns + the matching 128 `b` columns) so the SwiGLU
 // product pairs registers of the same lane.
 __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
-  using AOp = ROperand<BM>;
-  using BOp = TOperand<BN>;
-  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  using AOp = Lin1A;
+  using BOp = Lin1B;
+  bf16* lds = dyn_lds();
   constexpr int BNH = BN / 2;
   const int nb = (p.H + BNH - 1) / BNH;
   const TileCoord tc = decode_tile(p.table, nb);
@@ -42,8 +45,8 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
     return p.x + (int64_t)p.idx[tc.row0 + rr] * D;
   });
   B.init([&](int c) -> const bf16* {
-    const int half = c / BNH, j = j0 + (c % BNH);
-    return j < H ? w + half * H + j : nullptr;
+    const int half = c / BNH, j = min(j0 + (c % BNH), H - 8);
+    return w + half * H + j;
   }, 2 * H);
 
   const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
@@ -94,9 +97,9 @@ struct Lin2Args {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
-  using AOp = ROperand<BM>;
-  using BOp = TOperand<BN>;
-  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  using AOp = Lin1A;
+  using BOp = Lin1B;
+  bf16* lds = dyn_lds();
   const int D = p.D, H = p.H;
   const int nb = (D + BN - 1) / BN;
   const TileCoord tc = decode_tile(p.table, nb);
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
   AOp A;
   BOp B;
   A.init([&](int r) { return p.h + ((int64_t)tc.row0 + min(r, tc.rows - 1)) * H; });
-  B.init([&](int c) -> const bf16* { return d0 + c < D ? w + d0 + c : nullptr; }, D);
+  B.init([&](int c) -> const bf16* { return w + min(d0 + c, D - 8); }, D);
 
   const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
   const int m_org[FM] = {wm * 64, wm * 64 + 32};
@@ -192,7 +195,9 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H};
   const unsigned grid = grid_for(Msum, N, cdiv64(H, BN / 2));
-  lin1_swiglu_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  static std::once_flag once;
+  allow_lds(lin1_swiglu_kernel, kFwdLds, once);
+  lin1_swiglu_kernel<<<grid, kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -210,7 +215,9 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, co
   Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H};
   const unsigned grid = grid_for(Msum, N, cdiv64(D, BN));
-  lin2_scale_kernel<<<grid, kThreads, 0, (hipStream_t)stream>>>(a);
+  static std::once_flag once;
+  allow_lds(lin2_scale_kernel, kFwdLds, once);
+  lin2_scale_kernel<<<grid, kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

@@ -1,7 +1,8 @@
 // Weight-gradient grouped GEMM: GW[i] = A_i^T . B_i, contracting over the sorted
 // rows of expert i.  Both operands are stored [row][feature], i.e. k-strided, so
 // both go through the LDS transpose read.  Rows may be gathered through an index
-// (x and G_y are never materialised in sorted order).
+// (x and G_y are never materialised in sorted order); rows past the expert's last
+// one read a block of zeros.
 #include "gemm_tile.hpp"
 
 namespace momoe {
@@ -11,61 +12,9 @@ constexpr int BX = 128;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
 constexpr int FM = 2, FN = 4;
 
-// k-strided operand whose k-rows are the rows [row_begin,row_end) of an expert,
-// optionally gathered; rows past row_end are zero-filled.
-template <int COLS>
-struct TGatherOperand {
-  static constexpr int LD = COLS + 16;
-  static constexpr int CPR = COLS / 8;
-  static constexpr int KSTEP = kThreads / CPR;
-  static constexpr int NCH = kBK / KSTEP;
-  static constexpr int LDS_ELEMS = kBK * LD;
-  const bf16* base;  // column offset applied; nullptr when this thread's 8 columns are out of range
-  int64_t ld;
-  const int32_t* gather;
-  int row_begin, row_end;
-  int32_t rowid[NCH];
-  u32x4 stage[NCH];
-
-  __device__ __forceinline__ void fetch_rows(int kt) {
-    const int kr = threadIdx.x / CPR;
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int rr = row_begin + kt * kBK + kr + j * KSTEP;
-      int32_t id = -1;
-      if (rr < row_end) id = gather ? gather[rr] : rr;
-      rowid[j] = id;
-    }
-  }
-  __device__ __forceinline__ void init(const bf16* mat, int64_t ld_, const int32_t* gather_,
-                                       int col0, int ncols, int rb, int re) {
-    const int cc = threadIdx.x % CPR;
-    const int c = col0 + cc * 8;
-    base = c < ncols ? mat + c : nullptr;
-    ld = ld_;
-    gather = gather_;
-    row_begin = rb;
-    row_end = re;
-    fetch_rows(0);
-  }
-  // uses the row ids fetched for stage kt, then fetches those of stage kt+1
-  __device__ __forceinline__ void load(int kt) {
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      if (base != nullptr && rowid[j] >= 0) stage[j] = *(const u32x4*)(base + (int64_t)rowid[j] * ld);
-      else stage[j] = u32x4{0, 0, 0, 0};
-    }
-    fetch_rows(kt + 1);
-  }
-  __device__ __forceinline__ void store(bf16* lds) const {
-    const int cc = threadIdx.x % CPR, kr = threadIdx.x / CPR;
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) *(u32x4*)(lds + (kr + j * KSTEP) * LD + cc * 8) = stage[j];
-  }
-  static __device__ __forceinline__ bf16x8 frag(const bf16* lds, int c0, int kk) {
-    return TOperand<COLS>::frag(lds, c0, kk);
-  }
-};
+using OpA = TGatherDma<BX>;
+using OpB = TGatherDma<BY>;
+constexpr size_t kWgradLds = gemm_lds_bytes<OpA, OpB>();
 
 struct WgradArgs {
   const bf16* a;
@@ -84,9 +33,9 @@ struct WgradArgs {
 // XCDs and every tile of an expert runs on that one XCD, so the expert's rows are
 // fetched from HBM once and re-read from that XCD's L2.
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
-  using AOp = TGatherOperand<BX>;
-  using BOp = TGatherOperand<BY>;
-  __shared__ __attribute__((aligned(16))) bf16 lds[2 * (AOp::LDS_ELEMS + BOp::LDS_ELEMS)];
+  using AOp = OpA;
+  using BOp = OpB;
+  bf16* lds = dyn_lds();
   const int tpe = p.tiles_x * p.tiles_y;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int expert = (slot / tpe) * 8 + xcd;
@@ -147,6 +96,8 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
   if (blocks >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
               (bf16*)GW_NXY, (int)N, (int)X, (int)Y, tiles_x, tiles_y};
-  wgrad_kernel<<<(unsigned)blocks, kThreads, 0, (hipStream_t)stream>>>(a);
+  static std::once_flag once;
+  allow_lds(wgrad_kernel, kWgradLds, once);
+  wgrad_kernel<<<(unsigned)blocks, kThreads, kWgradLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
