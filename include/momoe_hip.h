@@ -34,7 +34,7 @@ extern "C" {
 #define MOMOE_ERR_LAUNCH 3      /* the HIP runtime refused a launch */
 
 /* rows per row-tile of the grouped GEMMs; the tile table must be built with it */
-#define MOMOE_TILE_ROWS 128
+#define MOMOE_TILE_ROWS 256
 /* column-block width of the partial row sums written by momoe_dgrad_h_swiglu_bwd */
 #define MOMOE_GS_BLOCK 256
 

@@ -16,7 +16,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;  // every GEMM workgroup is 4 wavefronts of 64
+constexpr int kThreads = 512;  // every GEMM workgroup is 8 wavefronts of 64: two per SIMD
+constexpr int kWaves = kThreads / 64;
 constexpr int kWave = 64;
 
 // Tile table layout (int32), written by the index build, read by the grouped GEMMs:
@@ -33,35 +34,46 @@ struct TileCoord {
   bool valid;
 };
 
-// Map the linear workgroup id to a (row tile, column block).  Workgroups are dealt
-// round-robin to the 8 XCDs, so id%8 selects the XCD; each XCD walks one contiguous
-// eighth of the (expert-major, column-block, row-tile-minor) sequence.  All tiles of
-// an expert therefore run on one XCD close together in time and share its L2 for
-// both the expert's weights and its token rows.
-__device__ __forceinline__ TileCoord decode_tile(const int* __restrict__ table, int nb) {
-  TileCoord tc;
-  tc.valid = false;
-  const int ntiles = table[0];
-  const int bm = table[1];
-  const int total = ntiles * nb;
-  const int chunk = (total + 7) >> 3;
-  const int bid = blockIdx.x;
-  const int xcd = bid & 7, slot = bid >> 3;
-  if (slot >= chunk) return tc;
-  const int q = xcd * chunk + slot;
-  if (q >= total) return tc;
-  const int* e = table + kTileHeader + 4 * (q / nb);
-  const int expert = e[0], first = e[1], rstart = e[2], mi = e[3];
-  const int nt = (mi + bm - 1) / bm;
-  const int qq = q - first * nb;
-  const int tl = qq % nt;
-  tc.tn = qq / nt;
-  tc.expert = expert;
-  tc.row0 = rstart + tl * bm;
-  tc.rows = min(bm, mi - tl * bm);
-  tc.valid = true;
-  return tc;
-}
+// Persistent-workgroup iterator over the (row tile, column block) pairs of a grouped GEMM.
+// Workgroups are dealt round-robin to the 8 XCDs, so id%8 selects the XCD; each XCD owns one
+// contiguous eighth of the (expert-major, column-block, row-tile-minor) sequence and its
+// workgroups walk it with a stride of gridDim/8.  All tiles of an expert therefore run on
+// one XCD close together in time and share its L2 for both the expert's weights and its
+// token rows.
+struct TileSched {
+  const int* table;
+  int nb, bm, total, chunk, xcd, pos, stride;
+
+  __device__ __forceinline__ TileSched(const int* table_, int nb_) : table(table_), nb(nb_) {
+    const int ntiles = *(const int __attribute__((address_space(4)))*)table;
+    bm = *(const int __attribute__((address_space(4)))*)(table + 1);
+    total = ntiles * nb;
+    chunk = (total + 7) >> 3;
+    xcd = blockIdx.x & 7;
+    pos = blockIdx.x >> 3;
+    stride = gridDim.x >> 3;
+  }
+  __device__ __forceinline__ TileCoord next() {
+    TileCoord tc;
+    tc.valid = false;
+    if (pos >= chunk) return tc;
+    const int q = xcd * chunk + pos;
+    pos += stride;
+    if (q >= total) return tc;
+    const int __attribute__((address_space(4)))* e =
+        (const int __attribute__((address_space(4)))*)(table + kTileHeader + 4 * (q / nb));
+    const int expert = e[0], first = e[1], rstart = e[2], mi = e[3];
+    const int nt = (mi + bm - 1) / bm;
+    const int qq = q - first * nb;
+    const int tl = qq % nt;
+    tc.tn = qq / nt;
+    tc.expert = expert;
+    tc.row0 = rstart + tl * bm;
+    tc.rows = min(bm, mi - tl * bm);
+    tc.valid = true;
+    return tc;
+  }
+};
 
 __device__ __forceinline__ float bf2f(bf16 v) { return (float)v; }
 __device__ __forceinline__ bf16 f2bf(float v) { return (bf16)v; }

@@ -8,11 +8,12 @@ namespace {
 
 constexpr int BM = MOMOE_TILE_ROWS;
 constexpr int BN = 256;
-constexpr int FM = 2, FN = 4;
+constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 rows x 64 columns
 static_assert(BN == MOMOE_GS_BLOCK, "gs_part blocks follow the column tile");
 using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
 using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
-constexpr size_t kBwdLds = gemm_lds_bytes<RowsA, RowsB>();
+using Ring = StageRing<RowsA, RowsB>;
+constexpr size_t kRedBytes = 4 * BM * sizeof(float);  // per-wave row sums of dL/ds
 
 struct DhArgs {
   const bf16* gy;
@@ -32,74 +33,103 @@ struct DhArgs {
 
 // u = G_y[idx] . Wl2^T is an "NT" GEMM: both operands are k-contiguous (k = D).
 __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
-  using AOp = RowsA;
-  using BOp = RowsB;
-  bf16* lds = dyn_lds();
   const int D = p.D, H = p.H;
-  const int nb = (H + BN - 1) / BN;
-  const TileCoord tc = decode_tile(p.table, nb);
+  const int KTILES = D / kBK;
+  Ring ring(dyn_lds());
+  float* red = (float*)(dyn_lds() + kStages * Ring::STAGE);  // [4 waves][BM], behind the stage ring
+  TileSched sched(p.table, (H + BN - 1) / BN);
+  RowsA A;
+  RowsB B;
+  auto start = [&](const TileCoord& t) {
+    const bf16* w = p.w2 + (int64_t)t.expert * H * D;
+    const int n0 = t.tn * BN;
+    A.init(p.gy, [&](int r) { return (uint32_t)p.idx[t.row0 + min(r, t.rows - 1)] * (uint32_t)(2 * D); });
+    B.init(w, [&](int r) { return (uint32_t)min(n0 + r, H - 1) * (uint32_t)(2 * D); });
+    gemm_issue_first(A, B, ring, KTILES);
+  };
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+
+  TileCoord tc = sched.next();
   if (!tc.valid) return;
-  const int n0 = tc.tn * BN;
-  const bf16* w = p.w2 + (int64_t)tc.expert * H * D;
+  start(tc);
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    gemm_rows<RowsA, RowsB, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
+    const TileCoord nx = sched.next();
+    if (nx.valid) start(nx);
 
-  AOp A;
-  BOp B;
-  A.init([&](int r) { return p.gy + (int64_t)p.idx[tc.row0 + min(r, tc.rows - 1)] * D; });
-  B.init([&](int r) { return w + (int64_t)min(n0 + r, H - 1) * D; });
-
-  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
-  const int m_org[FM] = {wm * 64, wm * 64 + 32};
-  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  f32x16 acc[FN][FM];
-  zero_acc<FM, FN>(acc);
-  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, D / kBK, lds, m_org, n_org);
-
-  __syncthreads();           // every wave is done with the LDS stages
-  float* red = (float*)lds;  // [2][BM]
+    const int n0 = tc.tn * BN;
+    float svs[FM];  // gate weights of this lane's rows, fetched ahead of the in-place stores
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int rloc = m_org[i] + acc_row();
-    float gsum = 0.0f;
-    if (rloc < tc.rows) {
-      const int64_t r = (int64_t)tc.row0 + rloc;
-      const float sv = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[r] * p.ssm];
-      const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
-      bf16* gzp = p.gz + r * 2 * H;
-      bf16* hsp = p.hs + r * H;
+    for (int i = 0; i < FM; ++i) {
+      const int rr = tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
+      svs[i] = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[rr] * p.ssm];
+    }
 #pragma unroll
-      for (int f = 0; f < FN; ++f) {
+    for (int i = 0; i < FM; ++i) {
+      const int rloc = m_org[i] + acc_row();
+      float gsum = 0.0f;
+      if (rloc < tc.rows) {
+        const int64_t r = (int64_t)tc.row0 + rloc;
+        const float sv = svs[i];
+        const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
+        bf16* gzp = p.gz + r * 2 * H;
+        bf16* hsp = p.hs + r * H;
+        // a|b of the whole fragment row are fetched before anything is stored: the stores go
+        // to the buffer the loads come from, so the compiler would otherwise serialise
+        // load -> compute -> store quad by quad, exposing the load latency 8 times
+        bf16x4 a4[FN][4], b4[FN][4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + n_org[f] + acc_col(q);
-          if (n >= H) continue;
-          const bf16x4 a4 = *(const bf16x4*)(abp + n);
-          const bf16x4 b4 = *(const bf16x4*)(abp + H + n);
-          float ga[4], gb[4], hv[4];
+        for (int f = 0; f < FN; ++f) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float a = (float)a4[e], b = (float)b4[e];
-            const float u = acc[f][i][4 * q + e];
-            const float sg = sigmoidf_fast(b);
-            const float hval = a * b * sg;
-            gsum += u * hval;
-            const float gh = sv * u;
-            ga[e] = gh * b * sg;
-            gb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
-            hv[e] = sv * hval;
+          for (int q = 0; q < 4; ++q) {
+            const int n = min(n0 + n_org[f] + acc_col(q), H - 4);
+            a4[f][q] = *(const bf16x4*)(abp + n);
+            b4[f][q] = *(const bf16x4*)(abp + H + n);
           }
-          store_bf16x4(gzp + n, ga[0], ga[1], ga[2], ga[3]);
-          store_bf16x4(gzp + H + n, gb[0], gb[1], gb[2], gb[3]);
-          store_bf16x4(hsp + n, hv[0], hv[1], hv[2], hv[3]);
+        }
+#pragma unroll
+        for (int f = 0; f < FN; ++f) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int n = n0 + n_org[f] + acc_col(q);
+            if (n >= H) continue;
+            float ga[4], gb[4], hv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a = (float)a4[f][q][e], b = (float)b4[f][q][e];
+              const float u = acc[f][i][4 * q + e];
+              const float sg = sigmoidf_fast(b);
+              const float hval = a * b * sg;
+              gsum += u * hval;
+              const float gh = sv * u;
+              ga[e] = gh * b * sg;
+              gb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
+              hv[e] = sv * hval;
+            }
+            store_bf16x4(gzp + n, ga[0], ga[1], ga[2], ga[3]);
+            store_bf16x4(gzp + H + n, gb[0], gb[1], gb[2], gb[3]);
+            store_bf16x4(hsp + n, hv[0], hv[1], hv[2], hv[3]);
+          }
         }
       }
+      gsum += __shfl_xor(gsum, 32);
+      if ((threadIdx.x & 63) < 32) red[wn * BM + rloc] = gsum;
     }
-    gsum += __shfl_xor(gsum, 32);
-    if ((threadIdx.x & 63) < 32) red[wn * BM + rloc] = gsum;
+    wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
+    __builtin_amdgcn_s_barrier();
+    if ((int)threadIdx.x < tc.rows)
+      p.gs_part[(int64_t)tc.tn * p.msum + tc.row0 + threadIdx.x] =
+          red[threadIdx.x] + red[BM + threadIdx.x] + red[2 * BM + threadIdx.x] +
+          red[3 * BM + threadIdx.x];
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();  // `red` is rewritten by the next tile
+    if (!nx.valid) break;
+    tc = nx;
   }
-  __syncthreads();
-  if (threadIdx.x < BM && (int)threadIdx.x < tc.rows)
-    p.gs_part[(int64_t)tc.tn * p.msum + tc.row0 + threadIdx.x] =
-        red[threadIdx.x] + red[BM + threadIdx.x];
 }
 
 struct DxArgs {
@@ -112,43 +142,52 @@ struct DxArgs {
 
 // gxs = gz . Wl1^T: contraction over the 2H contiguous columns of both operands.
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
-  using AOp = RowsA;
-  using BOp = RowsB;
-  bf16* lds = dyn_lds();
   const int D = p.D, H2 = 2 * p.H;
-  const int nb = (D + BN - 1) / BN;
-  const TileCoord tc = decode_tile(p.table, nb);
+  const int KTILES = H2 / kBK;
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (D + BN - 1) / BN);
+  RowsA A;
+  RowsB B;
+  auto start = [&](const TileCoord& t) {
+    const bf16* w = p.w1 + (int64_t)t.expert * D * H2;
+    const int d0 = t.tn * BN;
+    A.init(p.gz + (int64_t)t.row0 * H2, [&](int r) { return (uint32_t)(min(r, t.rows - 1) * 2 * H2); });
+    B.init(w, [&](int r) { return (uint32_t)min(d0 + r, D - 1) * (uint32_t)(2 * H2); });
+    gemm_issue_first(A, B, ring, KTILES);
+  };
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+
+  TileCoord tc = sched.next();
   if (!tc.valid) return;
-  const int d0 = tc.tn * BN;
-  const bf16* w = p.w1 + (int64_t)tc.expert * D * H2;
+  start(tc);
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    gemm_rows<RowsA, RowsB, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
+    const TileCoord nx = sched.next();
+    if (nx.valid) start(nx);
 
-  AOp A;
-  BOp B;
-  A.init([&](int r) { return p.gz + ((int64_t)tc.row0 + min(r, tc.rows - 1)) * H2; });
-  B.init([&](int r) { return w + (int64_t)min(d0 + r, D - 1) * H2; });
-
-  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
-  const int m_org[FM] = {wm * 64, wm * 64 + 32};
-  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  f32x16 acc[FN][FM];
-  zero_acc<FM, FN>(acc);
-  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, H2 / kBK, lds, m_org, n_org);
-
+    const int d0 = tc.tn * BN;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int rloc = m_org[i] + acc_row();
-    if (rloc >= tc.rows) continue;
-    bf16* out = p.gxs + ((int64_t)tc.row0 + rloc) * D;
+    for (int i = 0; i < FM; ++i) {
+      const int rloc = m_org[i] + acc_row();
+      if (rloc >= tc.rows) continue;
+      bf16* out = p.gxs + ((int64_t)tc.row0 + rloc) * D;
 #pragma unroll
-    for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int d = d0 + n_org[f] + acc_col(q);
-        if (d >= D) continue;
-        store_bf16x4(out + d, acc[f][i][4 * q], acc[f][i][4 * q + 1], acc[f][i][4 * q + 2],
-                     acc[f][i][4 * q + 3]);
+        for (int q = 0; q < 4; ++q) {
+          const int d = d0 + n_org[f] + acc_col(q);
+          if (d >= D) continue;
+          store_bf16x4(out + d, acc[f][i][4 * q], acc[f][i][4 * q + 1], acc[f][i][4 * q + 2],
+                       acc[f][i][4 * q + 3]);
+        }
       }
     }
+    if (!nx.valid) break;
+    tc = nx;
   }
 }
 
@@ -175,14 +214,10 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 inline int check_dims(int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum) {
   if (M <= 0 || D <= 0 || H <= 0 || N <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
   if (D % kBK != 0 || H % kBK != 0) return MOMOE_ERR_UNSUPPORTED;
-  if (Msum >= (1ll << 31) || M * D >= (1ll << 40) || D > (1 << 20) || H > (1 << 20))
+  // per-lane source offsets are 32-bit byte offsets from G_y / from an expert's weights
+  if (Msum >= (1ll << 31) || M * D * 2 >= (1ll << 32) || D * H * 4 >= (1ll << 32))
     return MOMOE_ERR_UNSUPPORTED;
   return MOMOE_OK;
-}
-
-inline unsigned grid_for(int64_t Msum, int64_t N, int64_t nb) {
-  const int64_t ub = max_row_tiles(Msum, N, BM) * nb;
-  return (unsigned)(cdiv64(ub, 8) * 8);
 }
 
 }  // namespace
@@ -208,10 +243,10 @@ extern "C" int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD, 
   DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m, idx_Msum,
            tile_table, (const bf16*)ab_save, Msave, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part,
            Msum, (int)D, (int)H};
-  const unsigned grid = grid_for(Msum, N, cdiv64(H, BN));
+  constexpr size_t lds = Ring::BYTES + kRedBytes;
   static std::once_flag once;
-  allow_lds(dgrad_h_swiglu_kernel, kBwdLds, once);
-  dgrad_h_swiglu_kernel<<<grid, kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_h_swiglu_kernel, lds, once);
+  dgrad_h_swiglu_kernel<<<persistent_grid(), kThreads, lds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -236,9 +271,8 @@ extern "C" int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H,
   if (st != MOMOE_OK) return st;
   DxArgs a{(const bf16*)gz_Msum2H, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
            (int)H};
-  const unsigned grid = grid_for(Msum, N, cdiv64(D, BN));
   static std::once_flag once;
-  allow_lds(dgrad_x_kernel, kBwdLds, once);
-  dgrad_x_kernel<<<grid, kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_x_kernel, Ring::BYTES, once);
+  dgrad_x_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
   return launch_status();
 }

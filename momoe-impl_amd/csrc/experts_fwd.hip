@@ -5,12 +5,12 @@
 namespace momoe {
 namespace {
 
-constexpr int BM = MOMOE_TILE_ROWS;  // 128 sorted rows per tile
-constexpr int BN = 256;              // output columns per tile
-constexpr int FM = 2, FN = 4;        // 2x2 waves, each 64 rows x 128 columns
-using Lin1A = RDma<BM>;              // token rows, k-contiguous
-using Lin1B = TDma<BN>;              // expert weights [k][col], k-strided
-constexpr size_t kFwdLds = gemm_lds_bytes<Lin1A, Lin1B>();
+constexpr int BM = MOMOE_TILE_ROWS;  // 256 sorted rows per tile
+constexpr int BN = 256;              // GEMM columns per tile
+constexpr int FM = 4, FN = 2;        // 2x4 waves, each 128 rows x 64 columns
+using RowsOp = RDma<BM>;             // token rows, k-contiguous
+using WeightOp = TDma;               // expert weights [k][col], k-strided
+using Ring = StageRing<RowsOp, WeightOp>;
 
 struct Lin1Args {
   const bf16* x;
@@ -23,56 +23,59 @@ struct Lin1Args {
   int D, H;
 };
 
-// Tile = 128 rows x (128 `a` columns + the matching 128 `b` columns) so the SwiGLU
-// product pairs registers of the same lane.
+// Tile = 256 rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
+// columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
 __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
-  using AOp = Lin1A;
-  using BOp = Lin1B;
-  bf16* lds = dyn_lds();
   constexpr int BNH = BN / 2;
-  const int nb = (p.H + BNH - 1) / BNH;
-  const TileCoord tc = decode_tile(p.table, nb);
-  if (!tc.valid) return;
-  if (p.h == nullptr && (int64_t)tc.row0 + tc.rows <= p.ab_lo) return;
-  const int j0 = tc.tn * BNH;
   const int D = p.D, H = p.H;
-  const bf16* w = p.w1 + (int64_t)tc.expert * D * 2 * H;
+  const int KTILES = D / kBK;
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (H + BNH - 1) / BNH);
+  // without an h output only rows >= ab_lo are wanted: tiles entirely below are skipped
+  auto next_tile = [&]() {
+    TileCoord t = sched.next();
+    while (t.valid && p.h == nullptr && (int64_t)t.row0 + t.rows <= p.ab_lo) t = sched.next();
+    return t;
+  };
+  RowsOp A;
+  WeightOp B;
+  auto start = [&](const TileCoord& t) {
+    const bf16* w = p.w1 + (int64_t)t.expert * D * 2 * H;
+    const int j0 = t.tn * BNH;
+    A.init(p.x, [&](int r) { return (uint32_t)p.idx[t.row0 + min(r, t.rows - 1)] * (uint32_t)(2 * D); });
+    B.init(w, [&](int c) { return (c / BNH) * H + min(j0 + (c % BNH), H - 8); }, 2 * H);
+    gemm_issue_first(A, B, ring, KTILES);
+  };
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 32, BNH + wn * 32};
 
-  AOp A;
-  BOp B;
-  A.init([&](int r) {
-    const int rr = min(r, tc.rows - 1);
-    return p.x + (int64_t)p.idx[tc.row0 + rr] * D;
-  });
-  B.init([&](int c) -> const bf16* {
-    const int half = c / BNH, j = min(j0 + (c % BNH), H - 8);
-    return w + half * H + j;
-  }, 2 * H);
+  TileCoord tc = next_tile();
+  if (!tc.valid) return;
+  start(tc);
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    gemm_rows<RowsOp, WeightOp, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
+    const TileCoord nx = next_tile();
+    if (nx.valid) start(nx);  // the next tile's first stage travels during this epilogue
 
-  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
-  const int m_org[FM] = {wm * 64, wm * 64 + 32};
-  const int n_org[FN] = {wn * 64, wn * 64 + 32, BNH + wn * 64, BNH + wn * 64 + 32};
-  f32x16 acc[FN][FM];
-  zero_acc<FM, FN>(acc);
-  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, D / kBK, lds, m_org, n_org);
-
+    const int j0 = tc.tn * BNH;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int rloc = m_org[i] + acc_row();
-    if (rloc >= tc.rows) continue;
-    const int64_t r = (int64_t)tc.row0 + rloc;
-    const bool save = p.ab != nullptr && r >= p.ab_lo && r < p.ab_hi;
-#pragma unroll
-    for (int f = 0; f < FN / 2; ++f) {
+    for (int i = 0; i < FM; ++i) {
+      const int rloc = m_org[i] + acc_row();
+      if (rloc >= tc.rows) continue;
+      const int64_t r = (int64_t)tc.row0 + rloc;
+      const bool save = p.ab != nullptr && r >= p.ab_lo && r < p.ab_hi;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int j = j0 + wn * 64 + f * 32 + acc_col(q);
+        const int j = j0 + wn * 32 + acc_col(q);
         if (j >= H) continue;
         float a[4], b[4], hv[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          a[e] = acc[f][i][4 * q + e];
-          b[e] = acc[f + FN / 2][i][4 * q + e];
+          a[e] = acc[0][i][4 * q + e];
+          b[e] = acc[1][i][4 * q + e];
           hv[e] = a[e] * b[e] * sigmoidf_fast(b[e]);
         }
         if (p.h) store_bf16x4(p.h + r * H + j, hv[0], hv[1], hv[2], hv[3]);
@@ -82,6 +85,8 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
         }
       }
     }
+    if (!nx.valid) break;
+    tc = nx;
   }
 }
 
@@ -97,44 +102,59 @@ struct Lin2Args {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
-  using AOp = Lin1A;
-  using BOp = Lin1B;
-  bf16* lds = dyn_lds();
   const int D = p.D, H = p.H;
-  const int nb = (D + BN - 1) / BN;
-  const TileCoord tc = decode_tile(p.table, nb);
+  const int KTILES = H / kBK;
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (D + BN - 1) / BN);
+  RowsOp A;
+  WeightOp B;
+  auto start = [&](const TileCoord& t) {
+    const bf16* w = p.w2 + (int64_t)t.expert * H * D;
+    const int d0 = t.tn * BN;
+    A.init(p.h + (int64_t)t.row0 * H, [&](int r) { return (uint32_t)(min(r, t.rows - 1) * 2 * H); });
+    B.init(w, [&](int c) { return min(d0 + c, D - 8); }, D);
+    gemm_issue_first(A, B, ring, KTILES);
+  };
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+
+  TileCoord tc = sched.next();
   if (!tc.valid) return;
-  const int d0 = tc.tn * BN;
-  const bf16* w = p.w2 + (int64_t)tc.expert * H * D;
+  start(tc);
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    gemm_rows<RowsOp, WeightOp, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
+    const TileCoord nx = sched.next();
+    if (nx.valid) start(nx);
 
-  AOp A;
-  BOp B;
-  A.init([&](int r) { return p.h + ((int64_t)tc.row0 + min(r, tc.rows - 1)) * H; });
-  B.init([&](int c) -> const bf16* { return w + min(d0 + c, D - 8); }, D);
-
-  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
-  const int m_org[FM] = {wm * 64, wm * 64 + 32};
-  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  f32x16 acc[FN][FM];
-  zero_acc<FM, FN>(acc);
-  gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, H / kBK, lds, m_org, n_org);
-
+    const int d0 = tc.tn * BN;
+    float svs[FM];  // gate weights of this lane's rows
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int rloc = m_org[i] + acc_row();
-    if (rloc >= tc.rows) continue;
-    const int64_t r = (int64_t)tc.row0 + rloc;
-    const float sv = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[r] * p.ssm];
+    for (int i = 0; i < FM; ++i) {
+      const int rr = tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
+      svs[i] = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[rr] * p.ssm];
+    }
 #pragma unroll
-    for (int f = 0; f < FN; ++f) {
+    for (int i = 0; i < FM; ++i) {
+      const int rloc = m_org[i] + acc_row();
+      if (rloc >= tc.rows) continue;
+      const int64_t r = (int64_t)tc.row0 + rloc;
+      const float sv = svs[i];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int d = d0 + n_org[f] + acc_col(q);
-        if (d >= D) continue;
-        store_bf16x4(p.ys + r * D + d, acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
-                     acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv);
+      for (int f = 0; f < FN; ++f) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int d = d0 + n_org[f] + acc_col(q);
+          if (d >= D) continue;
+          store_bf16x4(p.ys + r * D + d, acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
+                       acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv);
+        }
       }
     }
+    if (!nx.valid) break;
+    tc = nx;
   }
 }
 
@@ -165,14 +185,10 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 inline int check_dims(int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum) {
   if (M <= 0 || D <= 0 || H <= 0 || N <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
   if (D % kBK != 0 || H % kBK != 0) return MOMOE_ERR_UNSUPPORTED;
-  if (Msum >= (1ll << 31) || M * D >= (1ll << 40) || D > (1 << 20) || H > (1 << 20))
+  // per-lane source offsets are 32-bit byte offsets from x / from an expert's weights
+  if (Msum >= (1ll << 31) || M * D * 2 >= (1ll << 32) || D * H * 4 >= (1ll << 32))
     return MOMOE_ERR_UNSUPPORTED;
   return MOMOE_OK;
-}
-
-inline unsigned grid_for(int64_t Msum, int64_t N, int64_t nb) {
-  const int64_t ub = max_row_tiles(Msum, N, BM) * nb;
-  return (unsigned)(cdiv64(ub, 8) * 8);
 }
 
 }  // namespace
@@ -194,10 +210,9 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   if (st != MOMOE_OK) return st;
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H};
-  const unsigned grid = grid_for(Msum, N, cdiv64(H, BN / 2));
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel, kFwdLds, once);
-  lin1_swiglu_kernel<<<grid, kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel, Ring::BYTES, once);
+  lin1_swiglu_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -214,10 +229,9 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, co
   if (st != MOMOE_OK) return st;
   Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H};
-  const unsigned grid = grid_for(Msum, N, cdiv64(D, BN));
   static std::once_flag once;
-  allow_lds(lin2_scale_kernel, kFwdLds, once);
-  lin2_scale_kernel<<<grid, kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin2_scale_kernel, Ring::BYTES, once);
+  lin2_scale_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

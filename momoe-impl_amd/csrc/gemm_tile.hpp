@@ -1,19 +1,33 @@
 // Workgroup-level bf16 GEMM building blocks for gfx950 (CDNA4).
 //
-// A workgroup of 4 wavefronts computes a BM x BN fp32 tile with
-// v_mfma_f32_32x32x16_bf16.  Both MFMA inputs want, per lane, 8 consecutive
-// k-values of one row (lane%32 = row, lane/32 = which group of 8 k's).  Two
-// kinds of operand tile feed that:
+// A workgroup of 8 wavefronts (two per SIMD: a lone wave leaves ~15% of the MFMA
+// issue slots empty) computes a 256 x 256 fp32 tile with
+// v_mfma_f32_32x32x16_bf16; each wave owns 128 x 64 of it in 8 accumulator
+// fragments (128 registers), one workgroup per CU.  Both MFMA inputs want, per lane, 8
+// consecutive k-values of one row (lane%32 = row, lane/32 = which group of 8
+// k's).  Two kinds of operand tile feed that:
 //
 //   RDma  - "k-contiguous": the operand is stored [row][k] in global memory.
 //           LDS stage [ROWS][32]; a fragment is one ds_read_b128.
 //   TDma  - "k-strided": the operand is stored [k][col] (the layout of the
 //           expert weights in the forward GEMMs, and of everything in the
-//           weight-gradient GEMMs).  LDS stage [32][COLS]; a fragment is two
+//           weight-gradient GEMMs).  LDS stage [32][256]; a fragment is two
 //           ds_read_b64_tr_b16, the gfx950 LDS transpose read: within each
 //           group of 16 lanes, lane i supplies the address of 4 consecutive
 //           columns of k-row i/4 (columns 4*(i%4)..+3) and receives column i
 //           of those 4 k-rows.
+//
+// Sizing facts measured on MI355X that shape this file:
+//   * LDS serves 16 lanes per clock: 256 B/clk for bank-conflict-free
+//     ds_read_b128, 128 B/clk for the transpose reads.
+//   * A CU streams at most ~27 B/clk from L2 and ~19 B/clk from beyond it, and tile
+//     traffic of this shape sustains ~17 B/clk (10.5 TB/s over the chip), so the tile
+//     is 256x256, the largest the register file holds, and even then the loads, not
+//     the MFMA pipe, set the pace: several stages must be in flight at all times.
+//   * Launching one 256x256 tile per workgroup costs ~25% in launch, pipeline fill
+//     and drain: workgroups are persistent and prefetch across tiles.
+//   * Rows of a ragged tile that do not exist are pointed at the last valid row: the 16
+//     lanes of a deposit then ask for one line instead of 16, which makes them nearly free.
 //
 // Global memory goes straight to LDS with global_load_lds_dwordx4 (no VGPR
 // staging): one wave instruction deposits 64 x 16 bytes contiguously.  Since
@@ -24,8 +38,12 @@
 // pointed at a clamped row/column (results masked at the store) or, where exact
 // zeros are needed along k, at a 16-byte block of zeros.
 //
-// The k-loop runs a 3-stage ring: while stage t is consumed, the loads of t+1
-// and t+2 are in flight; one s_barrier per stage.
+// The k-loop runs a ring of 4 stages of 32 k: while one stage is multiplied (2 MFMA
+// k-steps) the next three are in flight; one s_barrier per stage.  The fragments of
+// a stage's second k-step are read before the barrier that opens the next stage and
+// multiplied after it, so the matrix pipe stays fed while the first fragments of
+// the new stage travel from LDS.  At the end of a tile three buffers are free, so
+// the next tile's first three stages are requested before the epilogue starts.
 //
 // The MFMA is issued with the N-side fragment as its first input and the M-side
 // fragment as its second, so each lane ends up holding, for ONE tile row
@@ -39,24 +57,35 @@
 
 namespace momoe {
 
-constexpr int kBK = 32;     // k-extent of one LDS stage
-constexpr int kStages = 3;  // LDS ring depth
-constexpr int kChunkElems = 512;  // one wave-wide 16-byte-per-lane deposit = 1 KiB
+constexpr int kBK = 32;            // k-extent of one LDS stage
+constexpr int kKSteps = kBK / 16;  // MFMA k-steps per stage
+constexpr int kStages = 4;         // LDS ring depth
+constexpr int kChunkElems = 512;   // one wave-wide 16-byte-per-lane deposit = 1 KiB
 
 static __device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0, 0, 0, 0};
 
 __device__ __forceinline__ const bf16* zero_chunk() { return (const bf16*)kZeroChunk; }
 
-// 16 bytes per lane, global -> LDS.  `lds_wave_base` must be wave-uniform; lane L's bytes
-// land at lds_wave_base + 16*L.  Completion is tracked by vmcnt.  Issued as inline
+// 16 bytes per lane, global -> LDS.  `lds_wave_base` is a wave-uniform LDS byte address; lane
+// L's bytes land at lds_wave_base + 16*L.  Completion is tracked by vmcnt.  Issued as inline
 // assembly so that the compiler's own wait-count insertion does not know about the
-// transfer: with the builtin it forces vmcnt(0) in front of the LDS transpose reads,
-// which serialises the ring.  Ordering is therefore entirely manual: wait_vmcnt<>() +
-// s_barrier before a stage is read, s_barrier before it is overwritten.
-__device__ __forceinline__ void dma16(const bf16* g, bf16* lds_wave_base) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(
-      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) bf16*)lds_wave_base);
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_addr)
+// transfer: with the builtin it forces vmcnt(0) in front of the LDS transpose reads.
+// Ordering is therefore entirely manual: wait_vmcnt<>() + s_barrier before a stage is
+// read, s_barrier before it is overwritten.
+// LDS byte address of a pointer into LDS (done once per kernel; transfers then use integers)
+__device__ __forceinline__ uint32_t lds_address(bf16* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) bf16*)p;
+}
+__device__ __forceinline__ void dma16(const bf16* g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g),
+               "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
+               : "memory");
+}
+// same, the source given as a wave-uniform base plus a per-lane byte offset
+__device__ __forceinline__ void dma16(const bf16* uniform_base, uint32_t byte_offset,
+                                      uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_offset),
+               "s"(uniform_base), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                : "memory");
 }
 
@@ -65,6 +94,8 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
+// wait until every LDS / scalar-memory operation of this wave has returned
+__device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 
 __device__ __forceinline__ bf16x4 lds_read_tr4(const bf16* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)p);
@@ -74,62 +105,68 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 first, bf16x8 second, f32x16 c) 
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(first, second, c, 0, 0, 0);
 }
 
+// uniform (scalar-unit) load of an int32 that no kernel writes while this one runs
+__device__ __forceinline__ int32_t load_uniform(const int32_t* p) {
+  return *(const int32_t __attribute__((address_space(4)))*)p;
+}
+
 // ---- k-contiguous operand -------------------------------------------------------------
 // LDS stage: row r at elements [32r, 32r+32); its four 16-byte k-pieces are stored at
-// position piece ^ ((r>>1)&3), which spreads 8 consecutive rows of one k-piece over all banks.
+// position piece ^ ((r>>2)&3), so the 16 rows x 16 bytes that 16 consecutive lanes of a
+// fragment read touch cover 16 different 16-byte bank groups (256 bytes, one clock).
 template <int ROWS>
 struct RDma {
-  static_assert(ROWS % 64 == 0, "ROWS must be a multiple of 64");
-  static constexpr int NCH = ROWS / 64;  // deposits per wave per stage (16 rows each)
+  static_assert(ROWS % (16 * kWaves) == 0, "ROWS must be a multiple of 16 rows per wave");
+  static constexpr int NCH = ROWS / (16 * kWaves);  // deposits per wave per stage (16 rows each)
   static constexpr int LDS_ELEMS = ROWS * kBK;
-  const bf16* ptr[NCH];
+  const bf16* base;   // wave-uniform
+  uint32_t off[NCH];  // byte offset of this lane's piece of deposit j from `base`, at k=0
 
-  // rowptr(r) -> global pointer to k=0 of tile row r; must be readable for every r < ROWS
-  template <class RowPtr>
-  __device__ __forceinline__ void init(RowPtr rowptr) {
+  // row r of the tile starts at (char*)base_ + rowoff(r); every r < ROWS must be readable
+  template <class RowOff>
+  __device__ __forceinline__ void init(const bf16* base_, RowOff rowoff) {
     const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+    base = base_;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int row = (j * 4 + w) * 16 + (l >> 2);
-      const int piece = (l & 3) ^ ((row >> 1) & 3);
-      ptr[j] = rowptr(row) + piece * 8;
+      const int row = (j * kWaves + w) * 16 + (l >> 2);
+      const int piece = (l & 3) ^ ((row >> 2) & 3);
+      off[j] = rowoff(row) + piece * 16;
     }
   }
-  __device__ __forceinline__ void issue(int kt, bf16* stage) {
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
     const int w = threadIdx.x >> 6;
+    const bf16* b = base + kt * kBK;
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) dma16(ptr[j] + kt * kBK, stage + (j * 4 + w) * kChunkElems);
+    for (int j = 0; j < NCH; ++j) dma16(b, off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
   }
   // 32 rows starting at r0 (multiple of 32), k-step kk (16 k-values)
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int r0, int kk) {
     const int l = threadIdx.x & 63;
     const int row = r0 + (l & 31);
-    const int piece = (2 * kk + (l >> 5)) ^ ((row >> 1) & 3);
+    const int piece = (2 * kk + (l >> 5)) ^ ((row >> 2) & 3);
     return *(const bf16x8*)(stage + row * kBK + piece * 8);
   }
 };
 
-// ---- k-strided operand ----------------------------------------------------------------
-// LDS stage: k-row k at elements [COLS*k, COLS*(k+1)); 16-byte piece p of the row is stored
+// ---- k-strided operand, 256 columns -----------------------------------------------------
+// LDS stage: k-row k at elements [256k, 256k+256); 16-byte piece p of the row is stored
 // at position p ^ (2*(k&3)), so the 4 k-rows x 32 bytes that a 16-lane group of the
-// transpose read touches fall into 4 different bank quarters.
-template <int COLS>
+// transpose read touches fall into 4 different bank quarters.  A deposit covers two k-rows
+// (lanes 0-31 / 32-63); wave w deposits k-rows [4w, 4w+4).
 struct TLayout {
-  static_assert(COLS % 64 == 0 && COLS <= 512, "COLS must be 64..512, multiple of 64");
-  static constexpr int PPR = COLS / 8;          // pieces per k-row
-  static constexpr int RPC = 64 / PPR;          // k-rows per deposit
-  static constexpr int NCH = kBK / RPC / 4;     // deposits per wave per stage
-  static_assert(NCH >= 1, "tile too narrow");
+  static constexpr int COLS = 256;
+  static constexpr int NCH = kBK / (2 * kWaves);  // deposits per wave per stage
   static constexpr int LDS_ELEMS = kBK * COLS;
 
   // k-row and logical column (multiple of 8) fetched by this lane in deposit j
   static __device__ __forceinline__ void lane_piece(int j, int& krow, int& col) {
     const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
-    krow = (j * 4 + w) * RPC + l / PPR;
-    col = ((l % PPR) ^ (2 * (krow & 3))) * 8;
+    krow = w * (2 * NCH) + j * 2 + (l >> 5);
+    col = ((l & 31) ^ (2 * (krow & 3))) * 8;
   }
-  static __device__ __forceinline__ bf16* deposit(bf16* stage, int j) {
-    return stage + (j * 4 + (threadIdx.x >> 6)) * kChunkElems;
+  static __device__ __forceinline__ uint32_t deposit(uint32_t stage, int j) {
+    return stage + ((threadIdx.x >> 6) * NCH + j) * (kChunkElems * 2);
   }
   // 32 columns starting at c0 (multiple of 32), k-step kk (16 k-values)
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
@@ -144,29 +181,32 @@ struct TLayout {
 };
 
 // k-strided operand with a fixed pitch between k-rows (the expert weights)
-template <int COLS>
 struct TDma {
-  using L = TLayout<COLS>;
+  using L = TLayout;
   static constexpr int NCH = L::NCH;
   static constexpr int LDS_ELEMS = L::LDS_ELEMS;
-  const bf16* ptr[NCH];
+  const bf16* base;   // wave-uniform
+  uint32_t off[NCH];  // byte offset of this lane's piece of deposit j from `base`, at k=0
   int64_t kstride;
 
-  // colptr(c) -> global pointer to (k=0, tile column c), c a multiple of 8; columns outside
-  // the matrix must be clamped by the caller to something readable.
-  template <class ColPtr>
-  __device__ __forceinline__ void init(ColPtr colptr, int64_t ld) {
+  // coloff(c) -> element offset from base_ of (k=0, tile column c), c a multiple of 8;
+  // columns outside the matrix must be clamped by the caller to something readable.
+  // ld = elements between consecutive k-rows.
+  template <class ColOff>
+  __device__ __forceinline__ void init(const bf16* base_, ColOff coloff, int64_t ld) {
+    base = base_;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       int krow, col;
       L::lane_piece(j, krow, col);
-      ptr[j] = colptr(col) + (int64_t)krow * ld;
+      off[j] = (uint32_t)((coloff(col) + (int64_t)krow * ld) * 2);
     }
     kstride = (int64_t)kBK * ld;
   }
-  __device__ __forceinline__ void issue(int kt, bf16* stage) {
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+    const bf16* b = base + kt * kstride;
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) dma16(ptr[j] + kt * kstride, L::deposit(stage, j));
+    for (int j = 0; j < NCH; ++j) dma16(b, off[j], L::deposit(stage, j));
   }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
     return L::frag(stage, c0, kk);
@@ -174,29 +214,33 @@ struct TDma {
 };
 
 // k-strided operand whose k-rows are the sorted rows [row_begin,row_end) of one expert,
-// optionally gathered through an index; k-rows past row_end read the zero block.
-template <int COLS>
+// optionally gathered through an index; k-rows past row_end read the zero block.  The row
+// ids of a deposit are a wave-uniform pair: they are fetched with scalar loads one stage
+// ahead of their use.
 struct TGatherDma {
-  using L = TLayout<COLS>;
+  using L = TLayout;
   static constexpr int NCH = L::NCH;
   static constexpr int LDS_ELEMS = L::LDS_ELEMS;
   const bf16* mat;
   int64_t ld;
   const int32_t* gather;
   int row_begin, row_end;
-  int krow[NCH], col[NCH];
-  int32_t rowid[NCH];
+  int col[NCH];
+  int32_t id0[NCH], id1[NCH];
 
   __device__ __forceinline__ void fetch_rows(int kt) {
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int rr = row_begin + kt * kBK + krow[j];
-      int32_t id = -1;
-      if (rr < row_end) id = gather ? gather[rr] : rr;
-      rowid[j] = id;
+      const int rr = row_begin + kt * kBK + w * (2 * NCH) + j * 2;
+      int32_t a = -1, b = -1;
+      if (rr < row_end) a = gather ? load_uniform(gather + rr) : rr;
+      if (rr + 1 < row_end) b = gather ? load_uniform(gather + rr + 1) : rr + 1;
+      id0[j] = a;
+      id1[j] = b;
     }
   }
-  // columns [col0, col0+COLS) of the matrix; columns >= ncols are clamped to column 0
+  // columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
   __device__ __forceinline__ void init(const bf16* mat_, int64_t ld_, const int32_t* gather_,
                                        int col0, int ncols, int rb, int re) {
     mat = mat_;
@@ -206,86 +250,159 @@ struct TGatherDma {
     row_end = re;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      int c;
-      L::lane_piece(j, krow[j], c);
+      int krow, c;
+      L::lane_piece(j, krow, c);
       col[j] = col0 + c < ncols ? col0 + c : 0;
     }
     fetch_rows(0);
   }
   // must be called with kt = 0, 1, 2, ... in order: uses the row ids fetched for kt and
-  // starts fetching those of kt+1 before the deposits are issued
-  __device__ __forceinline__ void issue(int kt, bf16* stage) {
-    int32_t cur[NCH];
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) cur[j] = rowid[j];
-    fetch_rows(kt + 1);
+  // starts fetching those of kt+1
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+    const bool upper = (threadIdx.x & 63) >= 32;
+    const bf16* src[NCH];
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const bf16* src = cur[j] >= 0 ? mat + (int64_t)cur[j] * ld + col[j] : zero_chunk();
-      dma16(src, L::deposit(stage, j));
+      const int32_t id = upper ? id1[j] : id0[j];
+      src[j] = id >= 0 ? mat + (int64_t)id * ld + col[j] : zero_chunk();
     }
+    fetch_rows(kt + 1);
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) dma16(src[j], L::deposit(stage, j));
   }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
     return L::frag(stage, c0, kk);
   }
 };
 
-// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.
-// `m_org[fm]` / `n_org[fn]` are the LDS row (or column) origins of this wave's 32-wide
-// fragments inside the A / B stage.  On return other waves may still be reading LDS:
-// barrier before reusing it.
-template <class AOp, class BOp, int FM, int FN>
+// ---- the k-loop -----------------------------------------------------------------------------
+// Ring of kStages LDS stage buffers; `head` is the buffer of stage 0 of the current tile and
+// is carried from tile to tile by a persistent workgroup.
+template <class AOp, class BOp>
+struct StageRing {
+  static constexpr int STAGE = AOp::LDS_ELEMS + BOp::LDS_ELEMS;
+  static constexpr size_t BYTES = (size_t)kStages * STAGE * sizeof(bf16);
+  bf16* lds;
+  uint32_t addr;  // LDS byte address of `lds`
+  int head;
+  __device__ __forceinline__ explicit StageRing(bf16* lds_) : lds(lds_), addr(lds_address(lds_)), head(0) {}
+  __device__ __forceinline__ bf16* buf(int kt) const {
+    return lds + ((kt + head) & (kStages - 1)) * STAGE;
+  }
+  __device__ __forceinline__ uint32_t buf_addr(int kt) const {
+    return addr + ((kt + head) & (kStages - 1)) * (STAGE * 2);
+  }
+  __device__ __forceinline__ void advance(int ktiles) { head = (head + ktiles) & (kStages - 1); }
+};
+
+template <class AOp, class BOp>
+__device__ __forceinline__ void gemm_issue(AOp& A, BOp& B, StageRing<AOp, BOp>& ring, int kt) {
+  const uint32_t st = ring.buf_addr(kt);
+  A.issue(kt, st);
+  B.issue(kt, st + AOp::LDS_ELEMS * 2);
+}
+
+// Request the first three stages of a tile.  May be called right after the previous tile's
+// main loop, while other waves still multiply its last stage: the other three buffers were
+// released by that tile's last barrier.
+template <class AOp, class BOp>
+__device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp>& ring,
+                                                 int ktiles) {
+  gemm_issue(A, B, ring, 0);
+  if (ktiles > 1) gemm_issue(A, B, ring, 1);
+  if (ktiles > 2) gemm_issue(A, B, ring, 2);
+}
+
+// wait until the deposits of stage kt have landed, when the stages up to kt+2 have been
+// requested and everything older than stage kt is known to be complete
+template <int LOADS>
+__device__ __forceinline__ void wait_stage(int kt, int ktiles) {
+  static_assert(2 * LOADS <= 63, "vmcnt is a 6-bit counter");
+  if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
+  else if (kt + 1 < ktiles) wait_vmcnt<LOADS>();
+  else wait_vmcnt<0>();
+}
+
+// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.  The first three
+// stages must already have been requested with gemm_issue_first.  A wave whose rows of the
+// tile are all invalid passes ACTIVE=false: it takes part in the transfers and barriers but
+// reads no fragments and multiplies nothing.  On return the ring has advanced to the next
+// tile; three of its buffers are free, other waves may still be reading the fourth.
+template <class AOp, class BOp, int FM, int FN, bool ACTIVE>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
-                                              bf16* lds, const int (&m_org)[FM],
+                                              StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
                                               const int (&n_org)[FN]) {
-  constexpr int STAGE = AOp::LDS_ELEMS + BOp::LDS_ELEMS;
-  constexpr int LOADS = AOp::NCH + BOp::NCH;  // deposits per wave per stage
-  constexpr int KK = kBK / 16;
-  A.issue(0, lds);
-  B.issue(0, lds + AOp::LDS_ELEMS);
-  if (ktiles > 1) {
-    A.issue(1, lds + STAGE);
-    B.issue(1, lds + STAGE + AOp::LDS_ELEMS);
-  }
-  int stage = 0;
-  for (int kt = 0; kt < ktiles; ++kt) {
-    // stage kt of every wave has landed; everyone is done reading stage kt-1
-    if (kt + 1 < ktiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    const bf16* la = lds + stage * STAGE;
+  static_assert(kKSteps == 2 && kStages == 4, "written for 2 k-steps per stage, 4 stages");
+  constexpr int LOADS = AOp::NCH + BOp::NCH;
+  bf16x8 af[2][FM], bf[2][FN];
+  auto load_frags = [&](int kt, int kk) {
+    if (!ACTIVE) return;
+    const bf16* la = ring.buf(kt);
     const bf16* lb = la + AOp::LDS_ELEMS;
-    bf16x8 af[KK][FM], bf[KK][FN];
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
+    for (int i = 0; i < FM; ++i) af[kk][i] = AOp::frag(la, m_org[i], kk);
 #pragma unroll
-      for (int i = 0; i < FM; ++i) af[kk][i] = AOp::frag(la, m_org[i], kk);
+    for (int j = 0; j < FN; ++j) bf[kk][j] = BOp::frag(lb, n_org[j], kk);
+  };
+  auto multiply = [&](int kk) {
+    if (!ACTIVE) return;
 #pragma unroll
-      for (int j = 0; j < FN; ++j) bf[kk][j] = BOp::frag(lb, n_org[j], kk);
-    }
-    if (kt + 2 < ktiles) {
-      bf16* nx = lds + (stage == 0 ? 2 : stage - 1) * STAGE;
-      A.issue(kt + 2, nx);
-      B.issue(kt + 2, nx + AOp::LDS_ELEMS);
-    }
+    for (int j = 0; j < FN; ++j)
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int i = 0; i < FM; ++i) acc[j][i] = mfma32(bf[kk][j], af[kk][i], acc[j][i]);
-    stage = stage == kStages - 1 ? 0 : stage + 1;
+      for (int i = 0; i < FM; ++i) acc[j][i] = mfma32(bf[kk][j], af[kk][i], acc[j][i]);
+  };
+  // The scheduling fences keep the compiler from hoisting fragment reads across k-steps.
+  auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+
+  // Everything requested so far has landed (this also drains the previous tile's stores);
+  // every wave is done reading the previous tile, whose last buffer stage 3 will reuse.
+  wait_vmcnt<0>();
+  wait_lgkm0();
+  __builtin_amdgcn_s_barrier();
+  fence();
+  if (ktiles > 3) gemm_issue(A, B, ring, 3);
+  load_frags(0, 0);
+  fence();
+  // the last stage is peeled off so that the loop body has a single path: a branch around
+  // the barrier would make the compiler wait for the freshly issued fragment reads
+  for (int kt = 0; kt + 1 < ktiles; ++kt) {
+    load_frags(kt, 1);
+    multiply(0);
+    fence();
+    // stage kt+1 has landed; all LDS reads of stage kt have returned, so its buffer may be
+    // overwritten once every wave is past the barrier
+    wait_stage<LOADS>(kt + 1, ktiles);
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();
+    fence();
+    if (kt + 4 < ktiles) gemm_issue(A, B, ring, kt + 4);
+    fence();
+    load_frags(kt + 1, 0);
+    multiply(1);
+    fence();
   }
+  load_frags(ktiles - 1, 1);
+  multiply(0);
+  fence();
+  multiply(1);
+  fence();
+  ring.advance(ktiles);
+}
+
+// main loop for a wave that owns rows [wave_row0, wave_row0 + 32*FM) of a tile whose first
+// `rows` rows are valid
+template <class AOp, class BOp, int FM, int FN>
+__device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
+                                          StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
+                                          const int (&n_org)[FN], int rows) {
+  if (m_org[0] < rows) gemm_mainloop<AOp, BOp, FM, FN, true>(A, B, acc, ktiles, ring, m_org, n_org);
+  else gemm_mainloop<AOp, BOp, FM, FN, false>(A, B, acc, ktiles, ring, m_org, n_org);
 }
 
 // the workgroup's dynamic LDS (size given at launch)
 __device__ __forceinline__ bf16* dyn_lds() {
   extern __shared__ __attribute__((aligned(1024))) bf16 momoe_lds[];
   return momoe_lds;
-}
-
-template <class AOp, class BOp>
-constexpr size_t gemm_lds_bytes() {
-  return (size_t)kStages * (AOp::LDS_ELEMS + BOp::LDS_ELEMS) * sizeof(bf16);
 }
 
 // Kernels use more than the 64 KiB of LDS a launch gets by default: raise the limit once.
@@ -295,6 +412,16 @@ inline void allow_lds(Kernel kernel, size_t bytes, std::once_flag& once) {
     (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)bytes);
   });
+}
+
+// number of persistent workgroups: one per CU of the current device, rounded to the 8 XCDs
+inline int persistent_grid() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      cus <= 0)
+    cus = 256;
+  return (cus + 7) / 8 * 8;
 }
 
 template <int FM, int FN>

@@ -8,13 +8,10 @@
 namespace momoe {
 namespace {
 
-constexpr int BX = 128;  // output rows per tile (features of A)
+constexpr int BX = 256;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
-constexpr int FM = 2, FN = 4;
-
-using OpA = TGatherDma<BX>;
-using OpB = TGatherDma<BY>;
-constexpr size_t kWgradLds = gemm_lds_bytes<OpA, OpB>();
+constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 x 64
+using Ring = StageRing<TGatherDma, TGatherDma>;
 
 struct WgradArgs {
   const bf16* a;
@@ -29,50 +26,78 @@ struct WgradArgs {
   int tiles_x, tiles_y;
 };
 
-// 1-D grid.  id%8 is the XCD a workgroup lands on; experts are dealt round-robin to the
-// XCDs and every tile of an expert runs on that one XCD, so the expert's rows are
-// fetched from HBM once and re-read from that XCD's L2.
+struct WTile {
+  int expert, x0, y0, rb, re;
+  bool valid;
+};
+
+// Persistent workgroups.  id%8 is the XCD a workgroup lands on; experts are dealt
+// round-robin to the XCDs and every tile of an expert runs on that one XCD, so the
+// expert's rows are fetched from HBM once and re-read from that XCD's L2.
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
-  using AOp = OpA;
-  using BOp = OpB;
-  bf16* lds = dyn_lds();
+  Ring ring(dyn_lds());
   const int tpe = p.tiles_x * p.tiles_y;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int expert = (slot / tpe) * 8 + xcd;
-  if (expert >= p.N) return;
-  const int q = slot % tpe;
-  const int tx = q / p.tiles_y, ty = q % p.tiles_y;
-  const int rb = p.cumsums[expert], re = p.cumsums[expert + 1];
-  const int x0 = tx * BX, y0 = ty * BY;
+  const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
+  const int total = ((p.N + 7) >> 3) * tpe;  // tile slots of one XCD
+  int pos = blockIdx.x >> 3;
+  auto next_tile = [&]() {
+    WTile t;
+    t.valid = false;
+    while (pos < total) {
+      const int expert = (pos / tpe) * 8 + xcd, q = pos % tpe;
+      pos += stride;
+      if (expert >= p.N) continue;
+      t.expert = expert;
+      t.x0 = (q / p.tiles_y) * BX;
+      t.y0 = (q % p.tiles_y) * BY;
+      t.rb = load_uniform(p.cumsums + expert);
+      t.re = load_uniform(p.cumsums + expert + 1);
+      t.valid = true;
+      break;
+    }
+    return t;
+  };
+  TGatherDma A, B;
+  auto start = [&](const WTile& t) {
+    if (t.re <= t.rb) return;  // expert without rows: nothing to load, zeros are stored
+    A.init(p.a, p.lda, p.ga, t.x0, p.X, t.rb, t.re);
+    B.init(p.b, p.ldb, p.gb, t.y0, p.Y, t.rb, t.re);
+    gemm_issue_first(A, B, ring, (t.re - t.rb + kBK - 1) / kBK);
+  };
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
 
-  AOp A;
-  BOp B;
-  A.init(p.a, p.lda, p.ga, x0, p.X, rb, re);
-  B.init(p.b, p.ldb, p.gb, y0, p.Y, rb, re);
+  WTile tc = next_tile();
+  if (!tc.valid) return;
+  start(tc);
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    const int ktiles = (tc.re - tc.rb + kBK - 1) / kBK;
+    if (ktiles > 0)
+      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, true>(A, B, acc, ktiles, ring, m_org, n_org);
+    const WTile nx = next_tile();
+    if (nx.valid) start(nx);
 
-  const int wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
-  const int m_org[FM] = {wm * 64, wm * 64 + 32};
-  const int n_org[FN] = {wn * 128, wn * 128 + 32, wn * 128 + 64, wn * 128 + 96};
-  f32x16 acc[FN][FM];
-  zero_acc<FM, FN>(acc);
-  const int ktiles = (re - rb + kBK - 1) / kBK;
-  if (ktiles > 0) gemm_mainloop<AOp, BOp, FM, FN>(A, B, acc, ktiles, lds, m_org, n_org);
-
-  bf16* out = p.gw + (int64_t)expert * p.X * p.Y;
+    bf16* out = p.gw + (int64_t)tc.expert * p.X * p.Y;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int x = x0 + m_org[i] + acc_row();
-    if (x >= p.X) continue;
+    for (int i = 0; i < FM; ++i) {
+      const int x = tc.x0 + m_org[i] + acc_row();
+      if (x >= p.X) continue;
 #pragma unroll
-    for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f) {
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int y = y0 + n_org[f] + acc_col(qd);
-        if (y >= p.Y) continue;
-        store_bf16x4(out + (int64_t)x * p.Y + y, acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
-                     acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]);
+        for (int qd = 0; qd < 4; ++qd) {
+          const int y = tc.y0 + n_org[f] + acc_col(qd);
+          if (y >= p.Y) continue;
+          store_bf16x4(out + (int64_t)x * p.Y + y, acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
+                       acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]);
+        }
       }
     }
+    if (!nx.valid) break;
+    tc = nx;
   }
 }
 
@@ -92,12 +117,11 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
     return MOMOE_ERR_BAD_ARG;
   if (Msum >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
-  const int64_t blocks = cdiv64(N, 8) * 8 * tiles_x * tiles_y;
-  if (blocks >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  if (cdiv64(N, 8) * tiles_x * tiles_y >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
               (bf16*)GW_NXY, (int)N, (int)X, (int)Y, tiles_x, tiles_y};
   static std::once_flag once;
-  allow_lds(wgrad_kernel, kWgradLds, once);
-  wgrad_kernel<<<(unsigned)blocks, kThreads, kWgradLds, (hipStream_t)stream>>>(a);
+  allow_lds(wgrad_kernel, Ring::BYTES, once);
+  wgrad_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
   return launch_status();
 }

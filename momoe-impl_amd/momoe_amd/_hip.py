@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmomoe_hip.so")
 
-TILE_ROWS = 128
+TILE_ROWS = 256
 GS_BLOCK = 256
 
 if not os.path.exists(LIB_PATH):

@@ -34,8 +34,8 @@ def test_tiny_reference_config(save_percent):
     (1024, 512, 256, 16, 4, 0, None, 0),
     (1024, 512, 256, 16, 4, 0, None, 37),    # save boundary in the middle of a tile
     (999, 256, 320, 12, 3, 0, None, 100),    # ragged token count, H not a multiple of the column tile
-    (2048, 512, 352, 20, 6, 2, 1.8, 0),      # skew + shared experts, H = 11*32
-    (2048, 512, 352, 20, 6, 2, 1.8, 100),
+    (2048, 512, 384, 20, 6, 2, 1.8, 0),      # skew + shared experts, H = 1.5 column tiles
+    (2048, 512, 384, 20, 6, 2, 1.8, 100),
     (16, 256, 128, 32, 4, 0, None, 0),       # decode-sized: most experts empty
 ])
 def test_layer_parity(M, D, H, N, K, Ks, skew, sp):
