@@ -83,6 +83,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--save-percent", type=float, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 256 MiB device-to-device copy a few times, so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command contains a "
+                         "kernel of known traffic to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path "
@@ -102,6 +106,14 @@ def main():
     sd = s.T.contiguous().to(dev).T.requires_grad_()
     xd = x.to(dev, torch.bfloat16).reshape(B, S, D).requires_grad_()
     dyd = dy.to(dev, torch.bfloat16).reshape(B, S, D)
+
+    if args.calibrate_copy:
+        src = torch.empty(128 * 2**20, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def make_layer(sp):
         return momoe_amd.MoMoE(D, H, N, K, save_percent=sp, Wl1_ND2H=W1.to(dev), Wl2_NHD=W2.to(dev))

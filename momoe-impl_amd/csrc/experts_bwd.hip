@@ -13,7 +13,8 @@ static_assert(BN == MOMOE_GS_BLOCK, "gs_part blocks follow the column tile");
 using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
 using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
 using Ring = StageRing<RowsA, RowsB>;
-constexpr size_t kRedBytes = 4 * BM * sizeof(float);  // per-wave row sums of dL/ds
+constexpr size_t kBwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+static_assert(4 * BM * sizeof(float) <= kEpilogueLds, "the dL/ds row sums reuse the staging area");
 
 struct DhArgs {
   const bf16* gy;
@@ -36,7 +37,9 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
   const int D = p.D, H = p.H;
   const int KTILES = D / kBK;
   Ring ring(dyn_lds());
-  float* red = (float*)(dyn_lds() + kStages * Ring::STAGE);  // [4 waves][BM], behind the stage ring
+  bf16* epi = dyn_lds() + kStages * Ring::STAGE;
+  float* red = (float*)epi;  // [4 column waves][BM], shares the store staging area
+  RowStager<1> stage0(epi, 0), stage1(epi, 1);
   TileSched sched(p.table, (H + BN - 1) / BN);
   RowsA A;
   RowsB B;
@@ -61,63 +64,76 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
     const TileCoord nx = sched.next();
     if (nx.valid) start(nx);
 
-    const int n0 = tc.tn * BN;
+    const int n0 = tc.tn * BN + wn * 64;  // first hidden column of this wave
     float svs[FM];  // gate weights of this lane's rows, fetched ahead of the in-place stores
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       const int rr = tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
       svs[i] = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[rr] * p.ssm];
     }
+    float gsums[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int rloc = m_org[i] + acc_row();
+      gsums[i] = 0.0f;
+      if (m_org[i] >= tc.rows) continue;  // wave-uniform
+      const int rloc = min(m_org[i] + acc_row(), tc.rows - 1);
+      const int64_t r = (int64_t)tc.row0 + rloc;
+      const float sv = svs[i];
+      const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
       float gsum = 0.0f;
-      if (rloc < tc.rows) {
-        const int64_t r = (int64_t)tc.row0 + rloc;
-        const float sv = svs[i];
-        const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
-        bf16* gzp = p.gz + r * 2 * H;
-        bf16* hsp = p.hs + r * H;
-        // a|b of the whole fragment row are fetched before anything is stored: the stores go
-        // to the buffer the loads come from, so the compiler would otherwise serialise
-        // load -> compute -> store quad by quad, exposing the load latency 8 times
-        bf16x4 a4[FN][4], b4[FN][4];
 #pragma unroll
-        for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f) {
+        // a|b of the fragment are fetched before anything is stored: the stores go to the
+        // buffer the loads come from, so they could not be hoisted above them later
+        bf16x4 a4[4], b4[4], hv[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int n = min(n0 + n_org[f] + acc_col(q), H - 4);
-            a4[f][q] = *(const bf16x4*)(abp + n);
-            b4[f][q] = *(const bf16x4*)(abp + H + n);
-          }
+        for (int q = 0; q < 4; ++q) {
+          const int n = min(n0 + 32 * f + acc_col(q), H - 4);
+          a4[q] = *(const bf16x4*)(abp + n);
+          b4[q] = *(const bf16x4*)(abp + H + n);
         }
 #pragma unroll
-        for (int f = 0; f < FN; ++f) {
+        for (int q = 0; q < 4; ++q) {
+          const bool incol = n0 + 32 * f + acc_col(q) < H;
+          float va[4], vb[4], vh[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int n = n0 + n_org[f] + acc_col(q);
-            if (n >= H) continue;
-            float ga[4], gb[4], hv[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float a = (float)a4[f][q][e], b = (float)b4[f][q][e];
-              const float u = acc[f][i][4 * q + e];
-              const float sg = sigmoidf_fast(b);
-              const float hval = a * b * sg;
-              gsum += u * hval;
-              const float gh = sv * u;
-              ga[e] = gh * b * sg;
-              gb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
-              hv[e] = sv * hval;
-            }
-            store_bf16x4(gzp + n, ga[0], ga[1], ga[2], ga[3]);
-            store_bf16x4(gzp + H + n, gb[0], gb[1], gb[2], gb[3]);
-            store_bf16x4(hsp + n, hv[0], hv[1], hv[2], hv[3]);
+          for (int e = 0; e < 4; ++e) {
+            const float a = (float)a4[q][e], b = (float)b4[q][e];
+            const float u = acc[f][i][4 * q + e];
+            const float sg = sigmoidf_fast(b);
+            const float hval = a * b * sg;
+            gsum += incol ? u * hval : 0.0f;
+            const float gh = sv * u;
+            va[e] = gh * b * sg;
+            vb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
+            vh[e] = sv * hval;
           }
+          stage0.put(0, q, pack_bf16x4(va[0], va[1], va[2], va[3]));
+          stage1.put(0, q, pack_bf16x4(vb[0], vb[1], vb[2], vb[3]));
+          hv[q] = pack_bf16x4(vh[0], vh[1], vh[2], vh[3]);
         }
+        auto dst = [&](bf16* mat, int64_t ld, int col0) {
+          return [=](int row, int col) -> bf16* {
+            const int rl = m_org[i] + row;
+            if (rl >= tc.rows || n0 + 32 * f + col >= H) return nullptr;
+            return mat + ((int64_t)tc.row0 + rl) * ld + col0 + n0 + 32 * f + col;
+          };
+        };
+        stage0.flush(dst(p.gz, 2 * H, 0));
+        stage1.flush(dst(p.gz, 2 * H, H));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) stage0.put(0, q, hv[q]);
+        stage0.flush(dst(p.hs, H, 0));
       }
-      gsum += __shfl_xor(gsum, 32);
-      if ((threadIdx.x & 63) < 32) red[wn * BM + rloc] = gsum;
+      gsums[i] = m_org[i] + acc_row() < tc.rows ? gsum : 0.0f;
+    }
+    // every wave is done with its staging area before the row sums overwrite it
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const float g = gsums[i] + __shfl_xor(gsums[i], 32);
+      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = g;
     }
     wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
     __builtin_amdgcn_s_barrier();
@@ -158,6 +174,7 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
 
   TileCoord tc = sched.next();
   if (!tc.valid) return;
@@ -169,22 +186,21 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
     const TileCoord nx = sched.next();
     if (nx.valid) start(nx);
 
-    const int d0 = tc.tn * BN;
+    const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int rloc = m_org[i] + acc_row();
-      if (rloc >= tc.rows) continue;
-      bf16* out = p.gxs + ((int64_t)tc.row0 + rloc) * D;
+      if (m_org[i] >= tc.rows) break;
 #pragma unroll
-      for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int d = d0 + n_org[f] + acc_col(q);
-          if (d >= D) continue;
-          store_bf16x4(out + d, acc[f][i][4 * q], acc[f][i][4 * q + 1], acc[f][i][4 * q + 2],
-                       acc[f][i][4 * q + 3]);
-        }
-      }
+        for (int q = 0; q < 4; ++q)
+          stager.put(f, q, pack_bf16x4(acc[f][i][4 * q], acc[f][i][4 * q + 1],
+                                       acc[f][i][4 * q + 2], acc[f][i][4 * q + 3]));
+      stager.flush([&](int row, int col) -> bf16* {
+        const int rl = m_org[i] + row;
+        if (rl >= tc.rows || d0 + col >= D) return nullptr;
+        return p.gxs + ((int64_t)tc.row0 + rl) * D + d0 + col;
+      });
     }
     if (!nx.valid) break;
     tc = nx;
@@ -243,10 +259,9 @@ extern "C" int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD, 
   DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m, idx_Msum,
            tile_table, (const bf16*)ab_save, Msave, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part,
            Msum, (int)D, (int)H};
-  constexpr size_t lds = Ring::BYTES + kRedBytes;
   static std::once_flag once;
-  allow_lds(dgrad_h_swiglu_kernel, lds, once);
-  dgrad_h_swiglu_kernel<<<persistent_grid(), kThreads, lds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_h_swiglu_kernel, kBwdLds, once);
+  dgrad_h_swiglu_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -272,7 +287,7 @@ extern "C" int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H,
   DxArgs a{(const bf16*)gz_Msum2H, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
            (int)H};
   static std::once_flag once;
-  allow_lds(dgrad_x_kernel, Ring::BYTES, once);
-  dgrad_x_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_x_kernel, kBwdLds, once);
+  dgrad_x_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }

@@ -11,6 +11,7 @@ constexpr int FM = 4, FN = 2;        // 2x4 waves, each 128 rows x 64 columns
 using RowsOp = RDma<BM>;             // token rows, k-contiguous
 using WeightOp = TDma;               // expert weights [k][col], k-strided
 using Ring = StageRing<RowsOp, WeightOp>;
+constexpr size_t kFwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
 
 struct Lin1Args {
   const bf16* x;
@@ -49,6 +50,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
   const int n_org[FN] = {wn * 32, BNH + wn * 32};
+  RowStager<1> stager(dyn_lds() + kStages * Ring::STAGE);
 
   TileCoord tc = next_tile();
   if (!tc.valid) return;
@@ -60,29 +62,44 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
     const TileCoord nx = next_tile();
     if (nx.valid) start(nx);  // the next tile's first stage travels during this epilogue
 
-    const int j0 = tc.tn * BNH;
+    const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int rloc = m_org[i] + acc_row();
-      if (rloc >= tc.rows) continue;
-      const int64_t r = (int64_t)tc.row0 + rloc;
-      const bool save = p.ab != nullptr && r >= p.ab_lo && r < p.ab_hi;
+      if (m_org[i] >= tc.rows) break;  // wave-uniform: no valid row in this fragment row
+      float a[4][4], b[4][4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int j = j0 + wn * 32 + acc_col(q);
-        if (j >= H) continue;
-        float a[4], b[4], hv[4];
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          a[e] = acc[0][i][4 * q + e];
-          b[e] = acc[1][i][4 * q + e];
-          hv[e] = a[e] * b[e] * sigmoidf_fast(b[e]);
+          a[q][e] = acc[0][i][4 * q + e];
+          b[q][e] = acc[1][i][4 * q + e];
         }
-        if (p.h) store_bf16x4(p.h + r * H + j, hv[0], hv[1], hv[2], hv[3]);
-        if (save) {
-          store_bf16x4(p.ab + r * 2 * H + j, a[0], a[1], a[2], a[3]);
-          store_bf16x4(p.ab + r * 2 * H + H + j, b[0], b[1], b[2], b[3]);
-        }
+      // destination of 8 columns of tile row m_org[i]+row in a [*, ld] matrix, or nullptr
+      auto dst = [&](bf16* mat, int64_t ld, int col0, bool rows_lo_hi) {
+        return [=](int row, int col) -> bf16* {
+          const int rl = m_org[i] + row;
+          const int64_t r = (int64_t)tc.row0 + rl;
+          if (rl >= tc.rows || j0 + col >= H) return nullptr;
+          if (rows_lo_hi && (r < p.ab_lo || r >= p.ab_hi)) return nullptr;
+          return mat + r * ld + col0 + j0 + col;
+        };
+      };
+      if (p.h) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          stager.put(0, q, pack_bf16x4(a[q][0] * b[q][0] * sigmoidf_fast(b[q][0]),
+                                       a[q][1] * b[q][1] * sigmoidf_fast(b[q][1]),
+                                       a[q][2] * b[q][2] * sigmoidf_fast(b[q][2]),
+                                       a[q][3] * b[q][3] * sigmoidf_fast(b[q][3])));
+        stager.flush(dst(p.h, H, 0, false));
+      }
+      if (p.ab) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) stager.put(0, q, pack_bf16x4(a[q][0], a[q][1], a[q][2], a[q][3]));
+        stager.flush(dst(p.ab, 2 * H, 0, true));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) stager.put(0, q, pack_bf16x4(b[q][0], b[q][1], b[q][2], b[q][3]));
+        stager.flush(dst(p.ab, 2 * H, H, true));
       }
     }
     if (!nx.valid) break;
@@ -118,6 +135,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
 
   TileCoord tc = sched.next();
   if (!tc.valid) return;
@@ -129,7 +147,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
     const TileCoord nx = sched.next();
     if (nx.valid) start(nx);
 
-    const int d0 = tc.tn * BN;
+    const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
     float svs[FM];  // gate weights of this lane's rows
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -138,20 +156,19 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
     }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int rloc = m_org[i] + acc_row();
-      if (rloc >= tc.rows) continue;
-      const int64_t r = (int64_t)tc.row0 + rloc;
+      if (m_org[i] >= tc.rows) break;
       const float sv = svs[i];
 #pragma unroll
-      for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int d = d0 + n_org[f] + acc_col(q);
-          if (d >= D) continue;
-          store_bf16x4(p.ys + r * D + d, acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
-                       acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv);
-        }
-      }
+        for (int q = 0; q < 4; ++q)
+          stager.put(f, q, pack_bf16x4(acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
+                                       acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv));
+      stager.flush([&](int row, int col) -> bf16* {
+        const int rl = m_org[i] + row;
+        if (rl >= tc.rows || d0 + col >= D) return nullptr;
+        return p.ys + ((int64_t)tc.row0 + rl) * D + d0 + col;
+      });
     }
     if (!nx.valid) break;
     tc = nx;
@@ -211,8 +228,8 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel, Ring::BYTES, once);
-  lin1_swiglu_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel, kFwdLds, once);
+  lin1_swiglu_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -230,8 +247,8 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, co
   Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H};
   static std::once_flag once;
-  allow_lds(lin2_scale_kernel, Ring::BYTES, once);
-  lin2_scale_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
+  allow_lds(lin2_scale_kernel, kFwdLds, once);
+  lin2_scale_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

@@ -439,9 +439,60 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[FN][FM]) {
 __device__ __forceinline__ int acc_row() { return threadIdx.x & 31; }
 __device__ __forceinline__ int acc_col(int q) { return 8 * q + 4 * ((threadIdx.x & 63) >> 5); }
 
-__device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c, float d) {
-  bf16x4 v = {(bf16)a, (bf16)b, (bf16)c, (bf16)d};
-  *(bf16x4*)p = v;
+__device__ __forceinline__ bf16x4 pack_bf16x4(float a, float b, float c, float d) {
+  return bf16x4{(bf16)a, (bf16)b, (bf16)c, (bf16)d};
 }
+__device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c, float d) {
+  *(bf16x4*)p = pack_bf16x4(a, b, c, d);
+}
+
+// ---- coalesced epilogue stores ----------------------------------------------------------------
+// In the accumulator layout a lane owns 4 consecutive columns of one row, so a direct store
+// writes 8-byte pieces scattered over 32 rows and every 128-byte line is written in 8 partial
+// requests.  Instead each wave passes one 32-row fragment row at a time through a private LDS
+// area (32 rows x 32*NF columns) and reads it back with 16 bytes per lane, lanes running along
+// the rows: stores then cover whole lines.  Wave-private: no barrier is involved.
+constexpr int kStageBytesPerWave = 32 * 64 * 2;                  // NF = 2
+constexpr size_t kEpilogueLds = (size_t)kWaves * kStageBytesPerWave;
+
+template <int NF>
+struct RowStager {
+  static constexpr int CHUNKS = 4 * NF;        // 16-byte chunks per staged row
+  static constexpr int PITCH = 32 * NF;        // elements per staged row
+  static constexpr int PASSES = 32 * CHUNKS / 64;
+  bf16* st;  // this wave's staging area
+
+  // `slot` selects one of the 2/NF staging areas of this wave
+  __device__ __forceinline__ explicit RowStager(bf16* epilogue_lds, int slot = 0)
+      : st(epilogue_lds + (threadIdx.x >> 6) * (kStageBytesPerWave / 2) + slot * (32 * PITCH)) {}
+
+  // this lane's quad q of fragment f: row lane%32, columns 32f + 8q + 4*(lane/32) .. +3
+  __device__ __forceinline__ void put(int f, int q, bf16x4 v) {
+    const int l = threadIdx.x & 63, row = l & 31, half = l >> 5;
+    const int c = (4 * f + q) ^ (row & (CHUNKS - 1));
+    *(bf16x4*)(st + row * PITCH + c * 8 + half * 4) = v;
+  }
+  // pass p of PASSES: 16 bytes = columns [col, col+8) of row `row` (both relative to the
+  // fragment row: row in [0,32), col in [0, 32*NF))
+  __device__ __forceinline__ bf16x8 get(int p, int& row, int& col) const {
+    const int l = threadIdx.x & 63;
+    row = p * (64 / CHUNKS) + l / CHUNKS;
+    const int pc = l % CHUNKS;
+    col = (pc ^ (row & (CHUNKS - 1))) * 8;
+    return *(const bf16x8*)(st + row * PITCH + pc * 8);
+  }
+  // write everything put() since the last flush: dst(row, col) -> destination of 8 columns,
+  // or nullptr to drop them
+  template <class Dst>
+  __device__ __forceinline__ void flush(Dst dst) const {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      int row, col;
+      const bf16x8 v = get(p, row, col);
+      bf16* d = dst(row, col);
+      if (d != nullptr) *(bf16x8*)d = v;
+    }
+  }
+};
 
 }  // namespace momoe

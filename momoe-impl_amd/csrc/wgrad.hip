@@ -12,6 +12,7 @@ constexpr int BX = 256;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
 constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 x 64
 using Ring = StageRing<TGatherDma, TGatherDma>;
+constexpr size_t kWgradLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
 
 struct WgradArgs {
   const bf16* a;
@@ -67,6 +68,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
 
   WTile tc = next_tile();
   if (!tc.valid) return;
@@ -81,20 +83,20 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     if (nx.valid) start(nx);
 
     bf16* out = p.gw + (int64_t)tc.expert * p.X * p.Y;
+    const int y0 = tc.y0 + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const int x = tc.x0 + m_org[i] + acc_row();
-      if (x >= p.X) continue;
 #pragma unroll
-      for (int f = 0; f < FN; ++f) {
+      for (int f = 0; f < FN; ++f)
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const int y = tc.y0 + n_org[f] + acc_col(qd);
-          if (y >= p.Y) continue;
-          store_bf16x4(out + (int64_t)x * p.Y + y, acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
-                       acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]);
-        }
-      }
+        for (int qd = 0; qd < 4; ++qd)
+          stager.put(f, qd, pack_bf16x4(acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
+                                        acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]));
+      stager.flush([&](int row, int col) -> bf16* {
+        const int x = tc.x0 + m_org[i] + row;
+        if (x >= p.X || y0 + col >= p.Y) return nullptr;
+        return out + (int64_t)x * p.Y + y0 + col;
+      });
     }
     if (!nx.valid) break;
     tc = nx;
@@ -121,7 +123,7 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
               (bf16*)GW_NXY, (int)N, (int)X, (int)Y, tiles_x, tiles_y};
   static std::once_flag once;
-  allow_lds(wgrad_kernel, Ring::BYTES, once);
-  wgrad_kernel<<<persistent_grid(), kThreads, Ring::BYTES, (hipStream_t)stream>>>(a);
+  allow_lds(wgrad_kernel, kWgradLds, once);
+  wgrad_kernel<<<persistent_grid(), kThreads, kWgradLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
