@@ -148,7 +148,7 @@ class MoMoE(nn.Module):
         for the backward, 0..100.
         Wl1_ND2H / Wl2_NHD: optional initial weights, [N, D, 2H] and [N, H, D]; the first
         H columns of Wl1 are the linear half, the last H go through SiLU.
-    D and H must be multiples of 64.
+    D and H must be multiples of 32 (the k-depth of one GEMM stage).
     """
 
     def __init__(self, embedding_dim, intermediate_dim, num_experts, num_chosen_experts,
