@@ -20,8 +20,14 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None until measured for the kernel that is currently dominant.
-MEASURED_TRAFFIC_BYTES = {}
+# (profiles/momoe_layer_headline_{fetch,write}_size.txt; fetch scaled x2.0, write x1.0 by the
+# 256 MiB copy in the same runs); None for a kernel that has not been measured.
+MEASURED_TRAFFIC_BYTES = {
+    "momoe_lin1_swiglu_fwd": 2 * 1319890 * 1024 + 205571 * 1024,
+    "momoe_wgrad[Wl1]": 2 * 391517 * 1024 + 1048576 * 1024,
+    "momoe_dgrad_h_swiglu_bwd": 2 * 1024964 * 1024 + 519239 * 1024,
+    "momoe_dgrad_x": 2 * 1127312 * 1024 + 262144 * 1024,
+}
 
 
 def headline_inputs(M, D, H, N, K, seed=0):
