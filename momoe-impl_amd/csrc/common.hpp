@@ -40,38 +40,72 @@ struct TileCoord {
 // workgroups walk it with a stride of gridDim/8.  All tiles of an expert therefore run on
 // one XCD close together in time and share its L2 for both the expert's weights and its
 // token rows.
+// A tile is looked up in two steps so that the table read can travel while other work runs:
+// fetch() issues the scalar loads of the workgroup's next tile, resolve() does the arithmetic.
 struct TileSched {
+  struct Raw {
+    int q, expert, first, rstart, mi;
+    bool any;
+  };
   const int* table;
-  int nb, bm, total, chunk, xcd, pos, stride;
+  int nb, bm, begin, total, chunk, xcd, pos, stride;
 
-  __device__ __forceinline__ TileSched(const int* table_, int nb_) : table(table_), nb(nb_) {
+  // tiles before row tile `first_row_tile` (all its column blocks) are left out
+  __device__ __forceinline__ TileSched(const int* table_, int nb_, int first_row_tile = 0)
+      : table(table_), nb(nb_) {
     const int ntiles = *(const int __attribute__((address_space(4)))*)table;
     bm = *(const int __attribute__((address_space(4)))*)(table + 1);
+    begin = min(first_row_tile, ntiles) * nb;
     total = ntiles * nb;
-    chunk = (total + 7) >> 3;
+    chunk = (total - begin + 7) >> 3;
     xcd = blockIdx.x & 7;
     pos = blockIdx.x >> 3;
     stride = gridDim.x >> 3;
   }
-  __device__ __forceinline__ TileCoord next() {
-    TileCoord tc;
-    tc.valid = false;
-    if (pos >= chunk) return tc;
-    const int q = xcd * chunk + pos;
+  __device__ __forceinline__ Raw fetch() {
+    Raw r;
+    r.any = false;
+    if (pos >= chunk) return r;
+    const int q = begin + xcd * chunk + pos;
     pos += stride;
-    if (q >= total) return tc;
+    if (q >= total) return r;
     const int __attribute__((address_space(4)))* e =
         (const int __attribute__((address_space(4)))*)(table + kTileHeader + 4 * (q / nb));
-    const int expert = e[0], first = e[1], rstart = e[2], mi = e[3];
-    const int nt = (mi + bm - 1) / bm;
-    const int qq = q - first * nb;
+    r.q = q;
+    r.expert = e[0];
+    r.first = e[1];
+    r.rstart = e[2];
+    r.mi = e[3];
+    r.any = true;
+    return r;
+  }
+  __device__ __forceinline__ TileCoord resolve(const Raw& r) const {
+    TileCoord tc;
+    tc.valid = r.any;
+    if (!r.any) return tc;
+    const int nt = (r.mi + bm - 1) / bm;
+    const int qq = r.q - r.first * nb;
     const int tl = qq % nt;
     tc.tn = qq / nt;
-    tc.expert = expert;
-    tc.row0 = rstart + tl * bm;
-    tc.rows = min(bm, mi - tl * bm);
-    tc.valid = true;
+    tc.expert = r.expert;
+    tc.row0 = r.rstart + tl * bm;
+    tc.rows = min(bm, r.mi - tl * bm);
     return tc;
+  }
+  __device__ __forceinline__ TileCoord next() { return resolve(fetch()); }
+  // first row tile of the expert that holds sorted row `row` (number of row tiles if the row
+  // lies past the last expert): everything before it only has rows below `row`
+  static __device__ __forceinline__ int expert_tile_of_row(const int* table, int64_t row) {
+    const int ntiles = *(const int __attribute__((address_space(4)))*)table;
+    int lo = 0, hi = ntiles;  // experts of the row tiles before lo end at or below `row`
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      const int __attribute__((address_space(4)))* e =
+          (const int __attribute__((address_space(4)))*)(table + kTileHeader + 4 * mid);
+      if ((int64_t)e[2] + e[3] <= row) lo = mid + 1; else hi = mid;
+    }
+    if (lo >= ntiles) return ntiles;
+    return *(const int __attribute__((address_space(4)))*)(table + kTileHeader + 4 * lo + 1);
   }
 };
 

@@ -33,44 +33,39 @@ struct DhArgs {
 };
 
 // u = G_y[idx] . Wl2^T is an "NT" GEMM: both operands are k-contiguous (k = D).
-__global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
-  const int D = p.D, H = p.H;
-  const int KTILES = D / kBK;
-  Ring ring(dyn_lds());
-  bf16* epi = dyn_lds() + kStages * Ring::STAGE;
-  float* red = (float*)epi;  // [4 column waves][BM], shares the store staging area
-  RowStager<1> stage0(epi, 0), stage1(epi, 1);
-  TileSched sched(p.table, (H + BN - 1) / BN);
-  RowsA A;
-  RowsB B;
-  auto start = [&](const TileCoord& t) {
+struct DhProg {
+  struct Prep {
+    int32_t tok[RowsA::NCH];  // tokens of the rows this lane fetches
+    int32_t etok[FM];         // tokens of the rows this lane holds in the accumulators
+    float sv[FM];             // their gate weights
+  };
+  const DhArgs& p;
+  const int ktiles, wn;
+  const int (&m_org)[FM];
+  bf16* epi;  // store staging, later the row-sum exchange
+
+  __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
+#pragma unroll
+    for (int j = 0; j < RowsA::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsA::row_of(j), t.rows - 1)];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
+  }
+  __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) g.sv[i] = p.s[(int64_t)t.expert * p.ssn + (int64_t)g.etok[i] * p.ssm];
+  }
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep& g, RowsA& A, RowsB& B) const {
+    const int D = p.D, H = p.H;
     const bf16* w = p.w2 + (int64_t)t.expert * H * D;
     const int n0 = t.tn * BN;
-    A.init(p.gy, [&](int r) { return (uint32_t)p.idx[t.row0 + min(r, t.rows - 1)] * (uint32_t)(2 * D); });
-    B.init(w, [&](int r) { return (uint32_t)min(n0 + r, H - 1) * (uint32_t)(2 * D); });
-    gemm_issue_first(A, B, ring, KTILES);
-  };
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 64, wn * 64 + 32};
-
-  TileCoord tc = sched.next();
-  if (!tc.valid) return;
-  start(tc);
-  while (true) {
-    f32x16 acc[FN][FM];
-    zero_acc<FM, FN>(acc);
-    gemm_rows<RowsA, RowsB, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
-    const TileCoord nx = sched.next();
-    if (nx.valid) start(nx);
-
+    A.init(p.gy, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
+    B.init(w, [&](int r, int) { return (uint32_t)min(n0 + r, H - 1) * (uint32_t)(2 * D); });
+  }
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+    const int H = p.H;
+    float* red = (float*)epi;  // [4 column waves][BM], shares the store staging area
+    RowStager<1> stage0(epi, 0), stage1(epi, 1);
     const int n0 = tc.tn * BN + wn * 64;  // first hidden column of this wave
-    float svs[FM];  // gate weights of this lane's rows, fetched ahead of the in-place stores
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const int rr = tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
-      svs[i] = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[rr] * p.ssm];
-    }
     float gsums[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -78,7 +73,7 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
       if (m_org[i] >= tc.rows) continue;  // wave-uniform
       const int rloc = min(m_org[i] + acc_row(), tc.rows - 1);
       const int64_t r = (int64_t)tc.row0 + rloc;
-      const float sv = svs[i];
+      const float sv = g.sv[i];
       const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
       float gsum = 0.0f;
 #pragma unroll
@@ -113,7 +108,7 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
           hv[q] = pack_bf16x4(vh[0], vh[1], vh[2], vh[3]);
         }
         auto dst = [&](bf16* mat, int64_t ld, int col0) {
-          return [=](int row, int col) -> bf16* {
+          return [=, *this](int row, int col) -> bf16* {
             const int rl = m_org[i] + row;
             if (rl >= tc.rows || n0 + 32 * f + col >= H) return nullptr;
             return mat + ((int64_t)tc.row0 + rl) * ld + col0 + n0 + 32 * f + col;
@@ -132,8 +127,8 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      const float g = gsums[i] + __shfl_xor(gsums[i], 32);
-      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = g;
+      const float gg = gsums[i] + __shfl_xor(gsums[i], 32);
+      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = gg;
     }
     wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
     __builtin_amdgcn_s_barrier();
@@ -143,9 +138,17 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
           red[3 * BM + threadIdx.x];
     wait_lgkm0();
     __builtin_amdgcn_s_barrier();  // `red` is rewritten by the next tile
-    if (!nx.valid) break;
-    tc = nx;
   }
+};
+
+__global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (p.H + BN - 1) / BN);
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  DhProg prog{p, p.D / kBK, wn, m_org, dyn_lds() + kStages * Ring::STAGE};
+  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
 }
 
 struct DxArgs {
@@ -157,35 +160,24 @@ struct DxArgs {
 };
 
 // gxs = gz . Wl1^T: contraction over the 2H contiguous columns of both operands.
-__global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
-  const int D = p.D, H2 = 2 * p.H;
-  const int KTILES = H2 / kBK;
-  Ring ring(dyn_lds());
-  TileSched sched(p.table, (D + BN - 1) / BN);
-  RowsA A;
-  RowsB B;
-  auto start = [&](const TileCoord& t) {
+struct DxProg {
+  struct Prep {};
+  const DxArgs& p;
+  const int ktiles, wn;
+  const int (&m_org)[FM];
+  RowStager<2> stager;
+
+  __device__ __forceinline__ void gather(const TileCoord&, Prep&) const {}
+  __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, RowsA& A, RowsB& B) const {
+    const int D = p.D, H2 = 2 * p.H;
     const bf16* w = p.w1 + (int64_t)t.expert * D * H2;
     const int d0 = t.tn * BN;
-    A.init(p.gz + (int64_t)t.row0 * H2, [&](int r) { return (uint32_t)(min(r, t.rows - 1) * 2 * H2); });
-    B.init(w, [&](int r) { return (uint32_t)min(d0 + r, D - 1) * (uint32_t)(2 * H2); });
-    gemm_issue_first(A, B, ring, KTILES);
-  };
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
-
-  TileCoord tc = sched.next();
-  if (!tc.valid) return;
-  start(tc);
-  while (true) {
-    f32x16 acc[FN][FM];
-    zero_acc<FM, FN>(acc);
-    gemm_rows<RowsA, RowsB, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
-    const TileCoord nx = sched.next();
-    if (nx.valid) start(nx);
-
+    A.init(p.gz + (int64_t)t.row0 * H2, [&](int r, int) { return (uint32_t)(min(r, t.rows - 1) * 2 * H2); });
+    B.init(w, [&](int r, int) { return (uint32_t)min(d0 + r, D - 1) * (uint32_t)(2 * H2); });
+  }
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
+    const int D = p.D;
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -202,9 +194,17 @@ __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
         return p.gxs + ((int64_t)tc.row0 + rl) * D + d0 + col;
       });
     }
-    if (!nx.valid) break;
-    tc = nx;
   }
+};
+
+__global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (p.D + BN - 1) / BN);
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  DxProg prog{p, (2 * p.H) / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
 }
 
 __global__ __launch_bounds__(256) void gs_scatter_kernel(const float* __restrict__ part, int nparts,

@@ -26,42 +26,30 @@ struct Lin1Args {
 
 // Tile = 256 rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
 // columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
-__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
-  constexpr int BNH = BN / 2;
-  const int D = p.D, H = p.H;
-  const int KTILES = D / kBK;
-  Ring ring(dyn_lds());
-  TileSched sched(p.table, (H + BNH - 1) / BNH);
-  // without an h output only rows >= ab_lo are wanted: tiles entirely below are skipped
-  auto next_tile = [&]() {
-    TileCoord t = sched.next();
-    while (t.valid && p.h == nullptr && (int64_t)t.row0 + t.rows <= p.ab_lo) t = sched.next();
-    return t;
+struct Lin1Prog {
+  static constexpr int BNH = BN / 2;
+  struct Prep {
+    int32_t tok[RowsOp::NCH];  // tokens of the rows this lane fetches
   };
-  RowsOp A;
-  WeightOp B;
-  auto start = [&](const TileCoord& t) {
+  const Lin1Args& p;
+  const int ktiles, wn;
+  const int (&m_org)[FM];
+  RowStager<1> stager;
+
+  __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
+#pragma unroll
+    for (int j = 0; j < RowsOp::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsOp::row_of(j), t.rows - 1)];
+  }
+  __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep& g, RowsOp& A, WeightOp& B) const {
+    const int D = p.D, H = p.H;
     const bf16* w = p.w1 + (int64_t)t.expert * D * 2 * H;
     const int j0 = t.tn * BNH;
-    A.init(p.x, [&](int r) { return (uint32_t)p.idx[t.row0 + min(r, t.rows - 1)] * (uint32_t)(2 * D); });
+    A.init(p.x, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
     B.init(w, [&](int c) { return (c / BNH) * H + min(j0 + (c % BNH), H - 8); }, 2 * H);
-    gemm_issue_first(A, B, ring, KTILES);
-  };
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 32, BNH + wn * 32};
-  RowStager<1> stager(dyn_lds() + kStages * Ring::STAGE);
-
-  TileCoord tc = next_tile();
-  if (!tc.valid) return;
-  start(tc);
-  while (true) {
-    f32x16 acc[FN][FM];
-    zero_acc<FM, FN>(acc);
-    gemm_rows<RowsOp, WeightOp, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
-    const TileCoord nx = next_tile();
-    if (nx.valid) start(nx);  // the next tile's first stage travels during this epilogue
-
+  }
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
+    const int H = p.H;
     const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -76,7 +64,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
         }
       // destination of 8 columns of tile row m_org[i]+row in a [*, ld] matrix, or nullptr
       auto dst = [&](bf16* mat, int64_t ld, int col0, bool rows_lo_hi) {
-        return [=](int row, int col) -> bf16* {
+        return [=, *this](int row, int col) -> bf16* {
           const int rl = m_org[i] + row;
           const int64_t r = (int64_t)tc.row0 + rl;
           if (rl >= tc.rows || j0 + col >= H) return nullptr;
@@ -102,9 +90,20 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
         stager.flush(dst(p.ab, 2 * H, H, true));
       }
     }
-    if (!nx.valid) break;
-    tc = nx;
   }
+};
+
+__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
+  Ring ring(dyn_lds());
+  // without an h output only rows >= ab_lo are wanted: experts entirely below are skipped
+  const int first_tile =
+      p.h == nullptr && p.ab_lo > 0 ? TileSched::expert_tile_of_row(p.table, p.ab_lo) : 0;
+  TileSched sched(p.table, (p.H + Lin1Prog::BNH - 1) / Lin1Prog::BNH, first_tile);
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 32, Lin1Prog::BNH + wn * 32};
+  Lin1Prog prog{p, p.D / kBK, wn, m_org, RowStager<1>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
 }
 
 struct Lin2Args {
@@ -118,46 +117,38 @@ struct Lin2Args {
   int D, H;
 };
 
-__global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
-  const int D = p.D, H = p.H;
-  const int KTILES = H / kBK;
-  Ring ring(dyn_lds());
-  TileSched sched(p.table, (D + BN - 1) / BN);
-  RowsOp A;
-  WeightOp B;
-  auto start = [&](const TileCoord& t) {
+struct Lin2Prog {
+  struct Prep {
+    int32_t tok[FM];  // tokens of the rows this lane holds in the accumulators
+    float sv[FM];     // their gate weights
+  };
+  const Lin2Args& p;
+  const int ktiles, wn;
+  const int (&m_org)[FM];
+  RowStager<2> stager;
+
+  __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) g.tok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
+  }
+  __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) g.sv[i] = p.s[(int64_t)t.expert * p.ssn + (int64_t)g.tok[i] * p.ssm];
+  }
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, RowsOp& A, WeightOp& B) const {
+    const int D = p.D, H = p.H;
     const bf16* w = p.w2 + (int64_t)t.expert * H * D;
     const int d0 = t.tn * BN;
-    A.init(p.h + (int64_t)t.row0 * H, [&](int r) { return (uint32_t)(min(r, t.rows - 1) * 2 * H); });
+    A.init(p.h + (int64_t)t.row0 * H, [&](int r, int) { return (uint32_t)(min(r, t.rows - 1) * 2 * H); });
     B.init(w, [&](int c) { return min(d0 + c, D - 8); }, D);
-    gemm_issue_first(A, B, ring, KTILES);
-  };
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
-
-  TileCoord tc = sched.next();
-  if (!tc.valid) return;
-  start(tc);
-  while (true) {
-    f32x16 acc[FN][FM];
-    zero_acc<FM, FN>(acc);
-    gemm_rows<RowsOp, WeightOp, FM, FN>(A, B, acc, KTILES, ring, m_org, n_org, tc.rows);
-    const TileCoord nx = sched.next();
-    if (nx.valid) start(nx);
-
+  }
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+    const int D = p.D;
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
-    float svs[FM];  // gate weights of this lane's rows
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const int rr = tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
-      svs[i] = p.s[(int64_t)tc.expert * p.ssn + (int64_t)p.idx[rr] * p.ssm];
-    }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       if (m_org[i] >= tc.rows) break;
-      const float sv = svs[i];
+      const float sv = g.sv[i];
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
@@ -170,9 +161,17 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
         return p.ys + ((int64_t)tc.row0 + rl) * D + d0 + col;
       });
     }
-    if (!nx.valid) break;
-    tc = nx;
   }
+};
+
+__global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (p.D + BN - 1) / BN);
+  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
+  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  Lin2Prog prog{p, p.H / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
 }
 
 // out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.

@@ -60,6 +60,7 @@ namespace momoe {
 constexpr int kBK = 32;            // k-extent of one LDS stage
 constexpr int kKSteps = kBK / 16;  // MFMA k-steps per stage
 constexpr int kStages = 4;         // LDS ring depth
+constexpr int kFirst = 3;          // stages of a tile requested ahead of its main loop
 constexpr int kChunkElems = 512;   // one wave-wide 16-byte-per-lane deposit = 1 KiB
 
 static __device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0, 0, 0, 0};
@@ -122,16 +123,21 @@ struct RDma {
   const bf16* base;   // wave-uniform
   uint32_t off[NCH];  // byte offset of this lane's piece of deposit j from `base`, at k=0
 
-  // row r of the tile starts at (char*)base_ + rowoff(r); every r < ROWS must be readable
+  // tile row whose piece this lane fetches in deposit j
+  static __device__ __forceinline__ int row_of(int j) {
+    return (j * kWaves + (threadIdx.x >> 6)) * 16 + ((threadIdx.x & 63) >> 2);
+  }
+  // row r of the tile starts at (char*)base_ + rowoff(r, j), j being the deposit that fetches
+  // it for this lane (r = row_of(j)); every r < ROWS must be readable
   template <class RowOff>
   __device__ __forceinline__ void init(const bf16* base_, RowOff rowoff) {
-    const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l = threadIdx.x & 63;
     base = base_;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int row = (j * kWaves + w) * 16 + (l >> 2);
+      const int row = row_of(j);
       const int piece = (l & 3) ^ ((row >> 2) & 3);
-      off[j] = rowoff(row) + piece * 16;
+      off[j] = rowoff(row, j) + piece * 16;
     }
   }
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
@@ -286,13 +292,14 @@ struct StageRing {
   uint32_t addr;  // LDS byte address of `lds`
   int head;
   __device__ __forceinline__ explicit StageRing(bf16* lds_) : lds(lds_), addr(lds_address(lds_)), head(0) {}
-  __device__ __forceinline__ bf16* buf(int kt) const {
-    return lds + ((kt + head) & (kStages - 1)) * STAGE;
+  static __device__ __forceinline__ int slot(int s) {
+    return (kStages & (kStages - 1)) == 0 ? s & (kStages - 1) : (int)((unsigned)s % (unsigned)kStages);
   }
+  __device__ __forceinline__ bf16* buf(int kt) const { return lds + slot(kt + head) * STAGE; }
   __device__ __forceinline__ uint32_t buf_addr(int kt) const {
-    return addr + ((kt + head) & (kStages - 1)) * (STAGE * 2);
+    return addr + slot(kt + head) * (STAGE * 2);
   }
-  __device__ __forceinline__ void advance(int ktiles) { head = (head + ktiles) & (kStages - 1); }
+  __device__ __forceinline__ void advance(int ktiles) { head = slot(head + ktiles); }
 };
 
 template <class AOp, class BOp>
@@ -309,58 +316,68 @@ template <class AOp, class BOp>
 __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp>& ring,
                                                  int ktiles) {
   gemm_issue(A, B, ring, 0);
-  if (ktiles > 1) gemm_issue(A, B, ring, 1);
-  if (ktiles > 2) gemm_issue(A, B, ring, 2);
+#pragma unroll
+  for (int s = 1; s < kFirst; ++s)
+    if (ktiles > s) gemm_issue(A, B, ring, s);
 }
 
-// wait until the deposits of stage kt have landed, when the stages up to kt+2 have been
-// requested and everything older than stage kt is known to be complete
+// wait until the deposits of stage kt have landed, when the stages up to kt+kStages-2 have
+// been requested and everything older than stage kt is known to be complete
 template <int LOADS>
 __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
-  static_assert(2 * LOADS <= 63, "vmcnt is a 6-bit counter");
-  if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
+  static_assert((kStages - 2) * LOADS <= 63, "vmcnt is a 6-bit counter");
+  static_assert(kStages == 4 || kStages == 5, "wait ladder written for 4 or 5 stages");
+  if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS>();
+  else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
   else if (kt + 1 < ktiles) wait_vmcnt<LOADS>();
   else wait_vmcnt<0>();
 }
 
-// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.  The first three
-// stages must already have been requested with gemm_issue_first.  A wave whose rows of the
-// tile are all invalid passes ACTIVE=false: it takes part in the transfers and barriers but
-// reads no fragments and multiplies nothing.  On return the ring has advanced to the next
-// tile; three of its buffers are free, other waves may still be reading the fourth.
-template <class AOp, class BOp, int FM, int FN, bool ACTIVE>
+// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.  The first kFirst
+// stages must already have been requested with gemm_issue_first.  NA is the number of 32-row
+// fragment rows of this wave that hold valid rows (wave-uniform): the others are neither read
+// nor multiplied; with NA = 0 the wave only takes part in the transfers and barriers.
+// `hook` runs once, right after the barrier that opens the tile: loads issued there travel
+// under the whole main loop (they enter the vmcnt queue between two stages, which can only
+// make the stage waits err on the long side).  On return the ring has advanced to the next
+// tile; all buffers but the last stage's are free, other waves may still be reading that one.
+template <class AOp, class BOp, int FM, int FN, int NA, class Hook>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                               StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                              const int (&n_org)[FN]) {
-  static_assert(kKSteps == 2 && kStages == 4, "written for 2 k-steps per stage, 4 stages");
+                                              const int (&n_org)[FN], Hook hook) {
+  static_assert(kKSteps == 2, "written for 2 k-steps per stage");
+  static_assert(NA >= 0 && NA <= FM, "active fragment rows");
   constexpr int LOADS = AOp::NCH + BOp::NCH;
   bf16x8 af[2][FM], bf[2][FN];
   auto load_frags = [&](int kt, int kk) {
-    if (!ACTIVE) return;
+    if (NA == 0) return;
     const bf16* la = ring.buf(kt);
     const bf16* lb = la + AOp::LDS_ELEMS;
 #pragma unroll
-    for (int i = 0; i < FM; ++i) af[kk][i] = AOp::frag(la, m_org[i], kk);
+    for (int i = 0; i < NA; ++i) af[kk][i] = AOp::frag(la, m_org[i], kk);
 #pragma unroll
     for (int j = 0; j < FN; ++j) bf[kk][j] = BOp::frag(lb, n_org[j], kk);
   };
   auto multiply = [&](int kk) {
-    if (!ACTIVE) return;
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int i = 0; i < FM; ++i) acc[j][i] = mfma32(bf[kk][j], af[kk][i], acc[j][i]);
+      for (int i = 0; i < NA; ++i) acc[j][i] = mfma32(bf[kk][j], af[kk][i], acc[j][i]);
   };
   // The scheduling fences keep the compiler from hoisting fragment reads across k-steps.
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
   // Everything requested so far has landed (this also drains the previous tile's stores);
-  // every wave is done reading the previous tile, whose last buffer stage 3 will reuse.
+  // every wave is done reading the previous tile, whose last buffer the next stage will reuse.
   wait_vmcnt<0>();
   wait_lgkm0();
   __builtin_amdgcn_s_barrier();
   fence();
-  if (ktiles > 3) gemm_issue(A, B, ring, 3);
+#pragma unroll
+  for (int s = kFirst; s < kStages; ++s)
+    if (ktiles > s) gemm_issue(A, B, ring, s);
+  hook();
+  fence();
   load_frags(0, 0);
   fence();
   // the last stage is peeled off so that the loop body has a single path: a branch around
@@ -375,7 +392,7 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
     wait_lgkm0();
     __builtin_amdgcn_s_barrier();
     fence();
-    if (kt + 4 < ktiles) gemm_issue(A, B, ring, kt + 4);
+    if (kt + kStages < ktiles) gemm_issue(A, B, ring, kt + kStages);
     fence();
     load_frags(kt + 1, 0);
     multiply(1);
@@ -389,14 +406,19 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   ring.advance(ktiles);
 }
 
-// main loop for a wave that owns rows [wave_row0, wave_row0 + 32*FM) of a tile whose first
+// main loop for a wave that owns rows [m_org[0], m_org[0] + 32*FM) of a tile whose first
 // `rows` rows are valid
-template <class AOp, class BOp, int FM, int FN>
+template <class AOp, class BOp, int FM, int FN, class Hook>
 __device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                           StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                          const int (&n_org)[FN], int rows) {
-  if (m_org[0] < rows) gemm_mainloop<AOp, BOp, FM, FN, true>(A, B, acc, ktiles, ring, m_org, n_org);
-  else gemm_mainloop<AOp, BOp, FM, FN, false>(A, B, acc, ktiles, ring, m_org, n_org);
+                                          const int (&n_org)[FN], int rows, Hook hook) {
+  static_assert(FM == 4, "dispatch written for 4 fragment rows per wave");
+  const int na = __builtin_amdgcn_readfirstlane(min(FM, max(0, (rows - m_org[0] + 31) >> 5)));
+  if (na == 4) gemm_mainloop<AOp, BOp, FM, FN, 4>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else gemm_mainloop<AOp, BOp, FM, FN, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
 }
 
 // the workgroup's dynamic LDS (size given at launch)
@@ -446,6 +468,53 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
   *(bf16x4*)p = pack_bf16x4(a, b, c, d);
 }
 
+// ---- persistent tile loop ------------------------------------------------------------------------
+// Drives a workgroup through its (row tile, column block) pairs with everything a tile needs
+// from memory requested one tile ahead.  The tile program P supplies
+//   typename P::Prep                          per-tile values that come from loads
+//   gather(tile, prep)                        issue those loads; must not use their results
+//   late(tile, prep)                          loads that depend on gather()'s results: issued
+//                                             a tile later, under the tile's own main loop
+//   setup(tile, prep, A, B)                   operand set-up (may use gather()'s results)
+//   epilogue(tile, acc, prep)                 may use late()'s results
+//   ktiles                                    stages per tile
+// While tile t is multiplied: the table entry of tile t+2 and the gathered values of tile t+1
+// are in flight; after its main loop the first stages of tile t+1 are requested, then the
+// epilogue of tile t runs.
+template <int FM, int FN, class P, class AOp, class BOp>
+__device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp>& ring,
+                                              const int (&m_org)[FM], const int (&n_org)[FN]) {
+  TileCoord c0 = sched.next();
+  if (!c0.valid) return;
+  TileCoord c1 = sched.next();
+  typename P::Prep p0, p1;
+  AOp A;
+  BOp B;
+  prog.gather(c0, p0);
+  prog.setup(c0, p0, A, B);
+  gemm_issue_first(A, B, ring, prog.ktiles);
+  p1 = p0;
+  while (true) {
+    f32x16 acc[FN][FM];
+    zero_acc<FM, FN>(acc);
+    TileSched::Raw rn;
+    gemm_rows<AOp, BOp, FM, FN>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.rows, [&] {
+      prog.late(c0, p0);
+      if (c1.valid) prog.gather(c1, p1);
+      rn = sched.fetch();
+    });
+    if (c1.valid) {
+      prog.setup(c1, p1, A, B);
+      gemm_issue_first(A, B, ring, prog.ktiles);  // travels during this tile's epilogue
+    }
+    prog.epilogue(c0, acc, p0);
+    if (!c1.valid) break;
+    c0 = c1;
+    p0 = p1;
+    c1 = sched.resolve(rn);
+  }
+}
+
 // ---- coalesced epilogue stores ----------------------------------------------------------------
 // In the accumulator layout a lane owns 4 consecutive columns of one row, so a direct store
 // writes 8-byte pieces scattered over 32 rows and every 128-byte line is written in 8 partial
@@ -467,7 +536,7 @@ struct RowStager {
       : st(epilogue_lds + (threadIdx.x >> 6) * (kStageBytesPerWave / 2) + slot * (32 * PITCH)) {}
 
   // this lane's quad q of fragment f: row lane%32, columns 32f + 8q + 4*(lane/32) .. +3
-  __device__ __forceinline__ void put(int f, int q, bf16x4 v) {
+  __device__ __forceinline__ void put(int f, int q, bf16x4 v) const {
     const int l = threadIdx.x & 63, row = l & 31, half = l >> 5;
     const int c = (4 * f + q) ^ (row & (CHUNKS - 1));
     *(bf16x4*)(st + row * PITCH + c * 8 + half * 4) = v;

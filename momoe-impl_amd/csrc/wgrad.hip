@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     zero_acc<FM, FN>(acc);
     const int ktiles = (tc.re - tc.rb + kBK - 1) / kBK;
     if (ktiles > 0)
-      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, true>(A, B, acc, ktiles, ring, m_org, n_org);
+      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
     const WTile nx = next_tile();
     if (nx.valid) start(nx);
 
