@@ -25,7 +25,6 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "momoe_lin1_swiglu_fwd": 2 * 1319890 * 1024 + 205571 * 1024,
     "momoe_wgrad[Wl1]": 2 * 391517 * 1024 + 1048576 * 1024,
-    "momoe_dgrad_h_swiglu_bwd": 2 * 1024964 * 1024 + 519239 * 1024,
     "momoe_dgrad_x": 2 * 1127312 * 1024 + 262144 * 1024,
 }
 
@@ -47,7 +46,7 @@ def kernel_flops(D, H, msum):
     unit = float(D) * H * msum
     return {
         "momoe_lin1_swiglu_fwd": 4 * unit, "momoe_lin2_scale_fwd": 2 * unit,
-        "momoe_dgrad_h_swiglu_bwd": 2 * unit, "momoe_dgrad_x": 4 * unit,
+        "momoe_dgrad_h": 2 * unit, "momoe_lin1_swiglu_bwd": 4 * unit, "momoe_dgrad_x": 4 * unit,
         "momoe_wgrad[Wl2]": 2 * unit, "momoe_wgrad[Wl1]": 4 * unit,
     }
 

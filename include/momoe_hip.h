@@ -35,8 +35,8 @@ extern "C" {
 
 /* rows per row-tile of the grouped GEMMs; the tile table must be built with it */
 #define MOMOE_TILE_ROWS 256
-/* column-block width of the partial row sums written by momoe_dgrad_h_swiglu_bwd */
-#define MOMOE_GS_BLOCK 256
+/* column-block width of the partial row sums written by momoe_lin1_swiglu_bwd */
+#define MOMOE_GS_BLOCK 128
 
 int momoe_abi_version(void);
 const char* momoe_status_string(int status);
@@ -73,7 +73,7 @@ int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m
  * then only a|b is produced and row tiles entirely below ab_row_lo are skipped);
  * ab_rows bf16 [*,2H] indexed by the sorted row r (may be NULL): rows with
  * ab_row_lo <= r < ab_row_hi receive bf16(a)|bf16(b) (the selective save of
- * :141-145 with lo=0, hi=Msave; the backward recomputation with lo=Msave, hi=Msum).
+ * :141-145 with lo=0, hi=Msave).
  */
 int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
                           const int32_t* tile_table, void* h_MsumH,
@@ -96,26 +96,41 @@ int momoe_combine(const void* rows_MsumD, const int32_t* inv_MK, void* out_MD,
                   int64_t M, int64_t D, int64_t K, int64_t Msum, void* stream);
 
 /* ---- experts backward ----------------------------------------------------
- * momoe_dgrad_h_swiglu_bwd replaces making_nice_scatter_kernel (G_y part) and
- * swiglu_backward_kernel (momoe/momoe.py:298-350, 421-535), and produces the
- * gate-weight gradient that lin1_backward_kernel (:683-703) obtains from a
- * recomputed down projection:
- *   u    = G_y[idx[r]] @ Wl2[i]^T                      (fp32 accumulate over D)
- *   a,b  = row r of ab_save (r < Msave) or of gz (r >= Msave, written there
- *          beforehand by momoe_lin1_swiglu_fwd)
- *   G_h  = s[i,idx[r]] * u
- *   gz[r] = bf16( G_h*b*sig(b) | G_h*a*sig(b)*(1 + b*(1-sig(b))) )   (overwrites a|b)
- *   hs[r] = bf16( s * a*b*sig(b) )       (h pre-scaled by the gate weight for the Wl2 gradient)
- *   gs_part[p][r] = sum over the p-th block of MOMOE_GS_BLOCK hidden columns of u * a*b*sig(b)
+ * The reference's swiglu_backward_kernel (momoe/momoe.py:421-535) computes dL/dh = G_y.Wl2^T,
+ * recomputes a|b = x.Wl1 for rows that were not saved, and applies the SwiGLU backward, in one
+ * kernel; lin1_backward_kernel (:683-703) obtains the gate-weight gradient from a recomputed
+ * down projection.  Here the same results come from three entry points:
+ *
+ * momoe_dgrad_h:  u[r] = bf16( G_y[idx[r]] @ Wl2[i]^T )  (fp32 accumulate over D), the
+ *   gradient of h before the gate weight; u_MsumH bf16 [Msum,H] in sorted order.
+ *
+ * momoe_lin1_swiglu_bwd, for the sorted rows r >= row_lo (those without saved a|b):
+ *   a|b  = x[idx[r]] @ Wl1[i]   (fp32, kept in registers)
+ *   s    = s_NM[i, idx[r]],  sig = sigmoid(b)
+ *   gz[r] = bf16( s u b sig | s u a sig (1 + b (1 - sig)) )       [G_a | G_b]
+ *   hs[r] = bf16( s a b sig )       (h pre-scaled by the gate weight, for the Wl2 gradient)
+ *   gs_part[p][r] = sum over the p-th block of MOMOE_GS_BLOCK hidden columns of u a b sig
  * (sum_p gs_part[p][r] = G_y[idx[r]] . (h[r] @ Wl2[i]) = dL/ds, by associativity).
  * gs_part fp32 [ceil(H/MOMOE_GS_BLOCK)][Msum].
+ *
+ * momoe_swiglu_bwd_saved, for the rows r < Msave: the same from the saved a|b (bf16); the whole
+ * row sum goes to gs_part[0][r], zeros to the other parts.
  */
-int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD,
-                             const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
-                             const int32_t* idx_Msum, const int32_t* tile_table,
-                             const void* ab_save, int64_t Msave,
-                             void* gz_Msum2H, void* hs_MsumH, float* gs_part,
-                             int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32_t* idx_Msum,
+                  const int32_t* tile_table, void* u_MsumH,
+                  int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+
+int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
+                          const int32_t* tile_table, const void* u_MsumH,
+                          const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
+                          int64_t row_lo, void* gz_Msum2H, void* hs_MsumH, float* gs_part,
+                          int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
+
+int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH,
+                           const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
+                           const int32_t* idx_Msum, const int32_t* cumsums_N1, int64_t Msave,
+                           void* gz_Msum2H, void* hs_MsumH, float* gs_part, int64_t nparts,
+                           int64_t M, int64_t H, int64_t N, int64_t Msum, void* stream);
 
 /* momoe_gs_scatter: Gs_NM[i, idx[r]] = sum_p gs_part[p][r] for every sorted row r of
  * expert i (momoe/momoe.py:699-703 without atomics).  Gs_NM fp32 contiguous [N,M],

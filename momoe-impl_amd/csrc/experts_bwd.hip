@@ -1,6 +1,7 @@
-// Backward of the experts, data-gradient side: dL/dh fused with the SwiGLU
-// backward and the gate-weight gradient, dL/dx in sorted order, and the scatter
-// of the gate-weight gradient into [N, M].
+// Backward of the experts, data-gradient side: dL/dh (before the gate weight), the SwiGLU
+// backward for rows whose pre-activations were saved (the others get theirs in the epilogue of
+// the recomputing x.Wl1 GEMM), dL/dx in sorted order, and the scatter of the gate-weight
+// gradient into [N, M].
 #include "gemm_tile.hpp"
 
 namespace momoe {
@@ -9,26 +10,17 @@ namespace {
 constexpr int BM = MOMOE_TILE_ROWS;
 constexpr int BN = 256;
 constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 rows x 64 columns
-static_assert(BN == MOMOE_GS_BLOCK, "gs_part blocks follow the column tile");
 using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
 using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
 using Ring = StageRing<RowsA, RowsB>;
 constexpr size_t kBwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
-static_assert(4 * BM * sizeof(float) <= kEpilogueLds, "the dL/ds row sums reuse the staging area");
 
 struct DhArgs {
   const bf16* gy;
   const bf16* w2;
-  const float* s;
-  int64_t ssn, ssm;
   const int32_t* idx;
   const int32_t* table;
-  const bf16* ab_save;
-  int64_t msave;
-  bf16* gz;
-  bf16* hs;
-  float* gs_part;
-  int64_t msum;
+  bf16* u;
   int D, H;
 };
 
@@ -36,24 +28,17 @@ struct DhArgs {
 struct DhProg {
   struct Prep {
     int32_t tok[RowsA::NCH];  // tokens of the rows this lane fetches
-    int32_t etok[FM];         // tokens of the rows this lane holds in the accumulators
-    float sv[FM];             // their gate weights
   };
   const DhArgs& p;
   const int ktiles, wn;
   const int (&m_org)[FM];
-  bf16* epi;  // store staging, later the row-sum exchange
+  RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
     for (int j = 0; j < RowsA::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsA::row_of(j), t.rows - 1)];
-#pragma unroll
-    for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
   }
-  __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
-#pragma unroll
-    for (int i = 0; i < FM; ++i) g.sv[i] = p.s[(int64_t)t.expert * p.ssn + (int64_t)g.etok[i] * p.ssm];
-  }
+  __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
   __device__ __forceinline__ void setup(const TileCoord& t, const Prep& g, RowsA& A, RowsB& B) const {
     const int D = p.D, H = p.H;
     const bf16* w = p.w2 + (int64_t)t.expert * H * D;
@@ -61,94 +46,95 @@ struct DhProg {
     A.init(p.gy, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
     B.init(w, [&](int r, int) { return (uint32_t)min(n0 + r, H - 1) * (uint32_t)(2 * D); });
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
     const int H = p.H;
-    float* red = (float*)epi;  // [4 column waves][BM], shares the store staging area
-    RowStager<1> stage0(epi, 0), stage1(epi, 1);
     const int n0 = tc.tn * BN + wn * 64;  // first hidden column of this wave
-    float gsums[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      gsums[i] = 0.0f;
-      if (m_org[i] >= tc.rows) continue;  // wave-uniform
-      const int rloc = min(m_org[i] + acc_row(), tc.rows - 1);
-      const int64_t r = (int64_t)tc.row0 + rloc;
-      const float sv = g.sv[i];
-      const bf16* abp = r < p.msave ? p.ab_save + r * 2 * H : p.gz + r * 2 * H;
-      float gsum = 0.0f;
+      if (m_org[i] >= tc.rows) break;
 #pragma unroll
-      for (int f = 0; f < FN; ++f) {
-        // a|b of the fragment are fetched before anything is stored: the stores go to the
-        // buffer the loads come from, so they could not be hoisted above them later
-        bf16x4 a4[4], b4[4], hv[4];
+      for (int f = 0; f < FN; ++f)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = min(n0 + 32 * f + acc_col(q), H - 4);
-          a4[q] = *(const bf16x4*)(abp + n);
-          b4[q] = *(const bf16x4*)(abp + H + n);
-        }
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const bool incol = n0 + 32 * f + acc_col(q) < H;
-          float va[4], vb[4], vh[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float a = (float)a4[q][e], b = (float)b4[q][e];
-            const float u = acc[f][i][4 * q + e];
-            const float sg = sigmoidf_fast(b);
-            const float hval = a * b * sg;
-            gsum += incol ? u * hval : 0.0f;
-            const float gh = sv * u;
-            va[e] = gh * b * sg;
-            vb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
-            vh[e] = sv * hval;
-          }
-          stage0.put(0, q, pack_bf16x4(va[0], va[1], va[2], va[3]));
-          stage1.put(0, q, pack_bf16x4(vb[0], vb[1], vb[2], vb[3]));
-          hv[q] = pack_bf16x4(vh[0], vh[1], vh[2], vh[3]);
-        }
-        auto dst = [&](bf16* mat, int64_t ld, int col0) {
-          return [=, *this](int row, int col) -> bf16* {
-            const int rl = m_org[i] + row;
-            if (rl >= tc.rows || n0 + 32 * f + col >= H) return nullptr;
-            return mat + ((int64_t)tc.row0 + rl) * ld + col0 + n0 + 32 * f + col;
-          };
-        };
-        stage0.flush(dst(p.gz, 2 * H, 0));
-        stage1.flush(dst(p.gz, 2 * H, H));
-#pragma unroll
-        for (int q = 0; q < 4; ++q) stage0.put(0, q, hv[q]);
-        stage0.flush(dst(p.hs, H, 0));
-      }
-      gsums[i] = m_org[i] + acc_row() < tc.rows ? gsum : 0.0f;
+        for (int q = 0; q < 4; ++q)
+          stager.put(f, q, pack_bf16x4(acc[f][i][4 * q], acc[f][i][4 * q + 1],
+                                       acc[f][i][4 * q + 2], acc[f][i][4 * q + 3]));
+      stager.flush([&](int row, int col) -> bf16* {
+        const int rl = m_org[i] + row;
+        if (rl >= tc.rows || n0 + col >= H) return nullptr;
+        return p.u + ((int64_t)tc.row0 + rl) * H + n0 + col;
+      });
     }
-    // every wave is done with its staging area before the row sums overwrite it
-    wait_lgkm0();
-    __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-      const float gg = gsums[i] + __shfl_xor(gsums[i], 32);
-      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = gg;
-    }
-    wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
-    __builtin_amdgcn_s_barrier();
-    if ((int)threadIdx.x < tc.rows)
-      p.gs_part[(int64_t)tc.tn * p.msum + tc.row0 + threadIdx.x] =
-          red[threadIdx.x] + red[BM + threadIdx.x] + red[2 * BM + threadIdx.x] +
-          red[3 * BM + threadIdx.x];
-    wait_lgkm0();
-    __builtin_amdgcn_s_barrier();  // `red` is rewritten by the next tile
   }
 };
 
-__global__ __launch_bounds__(kThreads, 2) void dgrad_h_swiglu_kernel(DhArgs p) {
+__global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.H + BN - 1) / BN);
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DhProg prog{p, p.D / kBK, wn, m_org, dyn_lds() + kStages * Ring::STAGE};
+  DhProg prog{p, p.D / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
+}
+
+// SwiGLU backward for the sorted rows whose a|b were saved by the forward: one workgroup per
+// row, 8 hidden columns per thread and pass.
+struct SavedArgs {
+  const bf16* ab;
+  const bf16* u;
+  const float* s;
+  int64_t ssn, ssm;
+  const int32_t* idx;
+  const int32_t* cumsums;
+  bf16* gz;
+  bf16* hs;
+  float* gs_part;
+  int nparts;
+  int64_t msum;
+  int H, N;
+};
+
+__global__ __launch_bounds__(256) void swiglu_bwd_saved_kernel(SavedArgs p) {
+  const int64_t r = blockIdx.x;
+  const int H = p.H;
+  __shared__ float s_red[4];
+  // expert of row r: the i with cumsums[i] <= r < cumsums[i+1]
+  int lo = 0, hi = p.N;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (p.cumsums[mid] <= r) lo = mid; else hi = mid;
+  }
+  const float sv = p.s[(int64_t)lo * p.ssn + (int64_t)p.idx[r] * p.ssm];
+  const bf16* a_row = p.ab + r * 2 * H;
+  const bf16* u_row = p.u + r * H;
+  float gsum = 0.0f;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
+    const bf16x8 a8 = *(const bf16x8*)(a_row + c);
+    const bf16x8 b8 = *(const bf16x8*)(a_row + H + c);
+    const bf16x8 u8 = *(const bf16x8*)(u_row + c);
+    bf16x8 ga, gb, hv;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float a = (float)a8[e], b = (float)b8[e], u = (float)u8[e];
+      const float sg = sigmoidf_fast(b);
+      const float hval = a * b * sg;
+      gsum += u * hval;
+      const float gh = sv * u;
+      ga[e] = (bf16)(gh * b * sg);
+      gb[e] = (bf16)(gh * a * sg * (1.0f + b * (1.0f - sg)));
+      hv[e] = (bf16)(sv * hval);
+    }
+    *(bf16x8*)(p.gz + r * 2 * H + c) = ga;
+    *(bf16x8*)(p.gz + r * 2 * H + H + c) = gb;
+    *(bf16x8*)(p.hs + r * H + c) = hv;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) gsum += __shfl_xor(gsum, o);
+  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = gsum;
+  __syncthreads();
+  if (threadIdx.x == 0) p.gs_part[r] = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+  // the whole row sum sits in part 0
+  for (int q = 1 + threadIdx.x; q < p.nparts; q += 256) p.gs_part[(int64_t)q * p.msum + r] = 0.0f;
 }
 
 struct DxArgs {
@@ -241,27 +227,40 @@ inline int check_dims(int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum) 
 
 using namespace momoe;
 
-extern "C" int momoe_dgrad_h_swiglu_bwd(const void* Gy_MD, const void* Wl2_NHD, const float* s_NM,
-                                        int64_t s_stride_n, int64_t s_stride_m,
-                                        const int32_t* idx_Msum, const int32_t* tile_table,
-                                        const void* ab_save, int64_t Msave, void* gz_Msum2H,
-                                        void* hs_MsumH, float* gs_part, int64_t M, int64_t D,
-                                        int64_t H, int64_t N, int64_t Msum, void* stream) {
-  if (!Gy_MD || !Wl2_NHD || !s_NM || !idx_Msum || !tile_table || !gz_Msum2H || !hs_MsumH ||
-      !gs_part)
-    return MOMOE_ERR_BAD_ARG;
-  if (Msave < 0 || Msave > Msum || (Msave > 0 && !ab_save)) return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(Gy_MD) || !aligned16(Wl2_NHD) || ((uintptr_t)ab_save & 7) ||
-      ((uintptr_t)gz_Msum2H & 7) || ((uintptr_t)hs_MsumH & 7))
-    return MOMOE_ERR_BAD_ARG;
+extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32_t* idx_Msum,
+                             const int32_t* tile_table, void* u_MsumH, int64_t M, int64_t D,
+                             int64_t H, int64_t N, int64_t Msum, void* stream) {
+  if (!Gy_MD || !Wl2_NHD || !idx_Msum || !tile_table || !u_MsumH) return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(Gy_MD) || !aligned16(Wl2_NHD) || !aligned16(u_MsumH)) return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
-  DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m, idx_Msum,
-           tile_table, (const bf16*)ab_save, Msave, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part,
-           Msum, (int)D, (int)H};
+  DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, idx_Msum, tile_table, (bf16*)u_MsumH, (int)D,
+           (int)H};
   static std::once_flag once;
-  allow_lds(dgrad_h_swiglu_kernel, kBwdLds, once);
-  dgrad_h_swiglu_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_h_kernel, kBwdLds, once);
+  dgrad_h_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  return launch_status();
+}
+
+extern "C" int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH, const float* s_NM,
+                                      int64_t s_stride_n, int64_t s_stride_m,
+                                      const int32_t* idx_Msum, const int32_t* cumsums_N1,
+                                      int64_t Msave, void* gz_Msum2H, void* hs_MsumH,
+                                      float* gs_part, int64_t nparts, int64_t M, int64_t H,
+                                      int64_t N, int64_t Msum, void* stream) {
+  if (!ab_save || !u_MsumH || !s_NM || !idx_Msum || !cumsums_N1 || !gz_Msum2H || !hs_MsumH ||
+      !gs_part)
+    return MOMOE_ERR_BAD_ARG;
+  if (Msave < 0 || Msave > Msum || nparts <= 0 || M <= 0 || H <= 0 || N <= 0 || Msum <= 0)
+    return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_Msum2H) || !aligned16(hs_MsumH))
+    return MOMOE_ERR_BAD_ARG;
+  if (H % 8 != 0 || Msum >= (1ll << 31) || nparts > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
+  if (Msave == 0) return MOMOE_OK;
+  SavedArgs a{(const bf16*)ab_save, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m, idx_Msum,
+              cumsums_N1, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part, (int)nparts, Msum, (int)H,
+              (int)N};
+  swiglu_bwd_saved_kernel<<<(unsigned)Msave, 256, 0, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

@@ -22,25 +22,49 @@ struct Lin1Args {
   bf16* ab;
   int64_t ab_lo, ab_hi;
   int D, H;
+  // backward only (rows >= ab_lo): dL/dh without the gate weight, the gate weights, outputs
+  const bf16* u;
+  const float* s;
+  int64_t ssn, ssm;
+  bf16* gz;
+  bf16* hs;
+  float* gs_part;
+  int64_t msum;
 };
 
 // Tile = 256 rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
 // columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
+// BWD = false: forward / recomputation, writes h and/or a|b.  BWD = true: the a|b of the tile
+// stay in registers and go straight into the SwiGLU backward.
+template <bool BWD>
 struct Lin1Prog {
   static constexpr int BNH = BN / 2;
+  static_assert(BNH == MOMOE_GS_BLOCK, "gs_part blocks follow the hidden-column tile");
+  static_assert(4 * BM * sizeof(float) <= kEpilogueLds, "the dL/ds row sums reuse the staging area");
   struct Prep {
     int32_t tok[RowsOp::NCH];  // tokens of the rows this lane fetches
+    int32_t etok[BWD ? FM : 1];  // backward: tokens of the rows this lane holds in the accumulators
+    float sv[BWD ? FM : 1];      // and their gate weights
   };
   const Lin1Args& p;
   const int ktiles, wn;
   const int (&m_org)[FM];
-  RowStager<1> stager;
+  bf16* epi;  // store staging; in the backward also the row-sum exchange
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
     for (int j = 0; j < RowsOp::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsOp::row_of(j), t.rows - 1)];
+    if (BWD) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
+    }
   }
-  __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
+  __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
+    if (BWD) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) g.sv[i] = p.s[(int64_t)t.expert * p.ssn + (int64_t)g.etok[i] * p.ssm];
+    }
+  }
   __device__ __forceinline__ void setup(const TileCoord& t, const Prep& g, RowsOp& A, WeightOp& B) const {
     const int D = p.D, H = p.H;
     const bf16* w = p.w1 + (int64_t)t.expert * D * 2 * H;
@@ -48,8 +72,14 @@ struct Lin1Prog {
     A.init(p.x, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
     B.init(w, [&](int c) { return (c / BNH) * H + min(j0 + (c % BNH), H - 8); }, 2 * H);
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+    if (BWD) epilogue_bwd(tc, acc, g);
+    else epilogue_fwd(tc, acc);
+  }
+
+  __device__ __forceinline__ void epilogue_fwd(const TileCoord& tc, f32x16 (&acc)[FN][FM]) const {
     const int H = p.H;
+    RowStager<1> stager(epi);
     const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -91,18 +121,97 @@ struct Lin1Prog {
       }
     }
   }
+
+  // SwiGLU backward on the recomputed a|b (momoe/momoe.py:421-535): with u = dL/dh before the
+  // gate weight s,  G_a = s u b sig(b),  G_b = s u a sig(b) (1 + b (1 - sig(b))),
+  // hs = s a b sig(b),  and the partial row sum of u a b sig(b) over this tile's columns.
+  __device__ __forceinline__ void epilogue_bwd(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+    const int H = p.H;
+    RowStager<1> stager(epi);
+    float* red = (float*)epi;  // [4 column waves][BM]
+    const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
+    auto load_u = [&](int i, bf16x4 (&uq)[4]) {
+      const int64_t r = (int64_t)tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) uq[q] = *(const bf16x4*)(p.u + r * H + min(j0 + acc_col(q), H - 4));
+    };
+    RowStager<1> stager1(epi, 1);
+    float gsums[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      gsums[i] = 0.0f;
+      if (m_org[i] >= tc.rows) continue;  // wave-uniform
+      bf16x4 uq[4];
+      load_u(i, uq);
+      const float sv = g.sv[i];
+      float gsum = 0.0f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bool incol = j0 + acc_col(q) < H;
+        float va[4], vb[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = acc[0][i][4 * q + e], b = acc[1][i][4 * q + e];
+          const float u = (float)uq[q][e];
+          const float sg = sigmoidf_fast(b);
+          const float hval = a * b * sg;
+          gsum += incol ? u * hval : 0.0f;
+          const float gh = sv * u;
+          va[e] = gh * b * sg;
+          vb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
+          acc[0][i][4 * q + e] = sv * hval;  // a is not needed any more: keep hs in its place
+        }
+        stager.put(0, q, pack_bf16x4(va[0], va[1], va[2], va[3]));
+        stager1.put(0, q, pack_bf16x4(vb[0], vb[1], vb[2], vb[3]));
+      }
+      auto dst = [&](bf16* mat, int64_t ld, int col0) {
+        return [=, *this](int row, int col) -> bf16* {
+          const int rl = m_org[i] + row;
+          const int64_t r = (int64_t)tc.row0 + rl;
+          if (rl >= tc.rows || j0 + col >= H || r < p.ab_lo) return nullptr;
+          return mat + r * ld + col0 + j0 + col;
+        };
+      };
+      stager.flush(dst(p.gz, 2 * H, 0));
+      stager1.flush(dst(p.gz, 2 * H, H));
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        stager.put(0, q, pack_bf16x4(acc[0][i][4 * q], acc[0][i][4 * q + 1], acc[0][i][4 * q + 2],
+                                     acc[0][i][4 * q + 3]));
+      stager.flush(dst(p.hs, H, 0));
+      gsums[i] = m_org[i] + acc_row() < tc.rows ? gsum : 0.0f;
+    }
+    // every wave is done with its staging area before the row sums overwrite it
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const float gg = gsums[i] + __shfl_xor(gsums[i], 32);
+      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = gg;
+    }
+    wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
+    __builtin_amdgcn_s_barrier();
+    if ((int)threadIdx.x < tc.rows && (int64_t)tc.row0 + threadIdx.x >= p.ab_lo)
+      p.gs_part[(int64_t)tc.tn * p.msum + tc.row0 + threadIdx.x] =
+          red[threadIdx.x] + red[BM + threadIdx.x] + red[2 * BM + threadIdx.x] +
+          red[3 * BM + threadIdx.x];
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();  // `red` is rewritten by the next tile
+  }
 };
 
+template <bool BWD>
 __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
+  using Prog = Lin1Prog<BWD>;
   Ring ring(dyn_lds());
   // without an h output only rows >= ab_lo are wanted: experts entirely below are skipped
   const int first_tile =
       p.h == nullptr && p.ab_lo > 0 ? TileSched::expert_tile_of_row(p.table, p.ab_lo) : 0;
-  TileSched sched(p.table, (p.H + Lin1Prog::BNH - 1) / Lin1Prog::BNH, first_tile);
+  TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, first_tile);
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 32, Lin1Prog::BNH + wn * 32};
-  Lin1Prog prog{p, p.D / kBK, wn, m_org, RowStager<1>(dyn_lds() + kStages * Ring::STAGE)};
+  const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
+  Prog prog{p, p.D / kBK, wn, m_org, dyn_lds() + kStages * Ring::STAGE};
   run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
 }
 
@@ -219,16 +328,42 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
                                      int64_t N, int64_t Msum, void* stream) {
   if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || (!h_MsumH && !ab_rows))
     return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_MsumH & 7) ||
-      ((uintptr_t)ab_rows & 7))
+  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_MsumH & 15) ||
+      ((uintptr_t)ab_rows & 15))
     return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
-             (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H};
+             (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
+             nullptr, nullptr, 0, 0, nullptr, nullptr, nullptr, Msum};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel, kFwdLds, once);
-  lin1_swiglu_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel<false>, kFwdLds, once);
+  lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  return launch_status();
+}
+
+extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
+                                     const int32_t* idx_Msum, const int32_t* tile_table,
+                                     const void* u_MsumH, const float* s_NM, int64_t s_stride_n,
+                                     int64_t s_stride_m, int64_t row_lo, void* gz_Msum2H,
+                                     void* hs_MsumH, float* gs_part, int64_t M, int64_t D,
+                                     int64_t H, int64_t N, int64_t Msum, void* stream) {
+  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || !u_MsumH || !s_NM || !gz_Msum2H ||
+      !hs_MsumH || !gs_part)
+    return MOMOE_ERR_BAD_ARG;
+  if (row_lo < 0 || row_lo > Msum) return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)u_MsumH & 7) ||
+      !aligned16(gz_Msum2H) || !aligned16(hs_MsumH))
+    return MOMOE_ERR_BAD_ARG;
+  const int st = check_dims(M, D, H, N, Msum);
+  if (st != MOMOE_OK) return st;
+  if (row_lo == Msum) return MOMOE_OK;
+  Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, nullptr, nullptr,
+             row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
+             (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part, Msum};
+  static std::once_flag once;
+  allow_lds(lin1_swiglu_kernel<true>, kFwdLds, once);
+  lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

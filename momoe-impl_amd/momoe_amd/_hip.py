@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmomoe_hip.so")
 
 TILE_ROWS = 256
-GS_BLOCK = 256
+GS_BLOCK = 128
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
@@ -39,8 +39,11 @@ _SIGNATURES = {
     "momoe_lin2_scale_fwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64,
                                     _i64, _p]),
     "momoe_combine": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
-    "momoe_dgrad_h_swiglu_bwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _p, _p, _p,
-                                        _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_dgrad_h": (_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_lin1_swiglu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _p,
+                                     _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_swiglu_bwd_saved": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _i64, _p, _p, _p, _i64,
+                                      _i64, _i64, _i64, _i64, _p]),
     "momoe_gs_scatter": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _p]),
     "momoe_dgrad_x": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
@@ -168,13 +171,32 @@ def combine(rows_MsumD, inv_MK, out_MD):
 
 
 # ---------------------------------------------------------------- experts bwd
-def dgrad_h_swiglu_bwd(Gy_MD, Wl2_NHD, s_NM, idx, table, ab_save, Msave, gz, hs, gs_part):
+def dgrad_h(Gy_MD, Wl2_NHD, idx, table, u):
+    _need_cuda(Gy_MD, Wl2_NHD)
     M, D = Gy_MD.shape
     N, H, _ = Wl2_NHD.shape
-    _call("momoe_dgrad_h_swiglu_bwd", _ptr(Gy_MD), _ptr(Wl2_NHD), _ptr(s_NM), s_NM.stride(0),
-                                         s_NM.stride(1), _ptr(idx), _ptr(table), _ptr(ab_save),
-                                         Msave, _ptr(gz), _ptr(hs), _ptr(gs_part), M, D, H, N,
-                                         idx.numel(), _stream())
+    _call("momoe_dgrad_h", _ptr(Gy_MD), _ptr(Wl2_NHD), _ptr(idx), _ptr(table), _ptr(u), M, D, H, N,
+                              idx.numel(), _stream())
+
+
+def lin1_swiglu_bwd(x_MD, Wl1_ND2H, idx, table, u, s_NM, row_lo, gz, hs, gs_part):
+    _need_cuda(x_MD, Wl1_ND2H, u, s_NM)
+    M, D = x_MD.shape
+    N, _, H2 = Wl1_ND2H.shape
+    _call("momoe_lin1_swiglu_bwd", _ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(u),
+                                      _ptr(s_NM), s_NM.stride(0), s_NM.stride(1), row_lo, _ptr(gz),
+                                      _ptr(hs), _ptr(gs_part), M, D, H2 // 2, N, idx.numel(),
+                                      _stream())
+
+
+def swiglu_bwd_saved(ab_save, u, s_NM, idx, cumsums, Msave, gz, hs, gs_part):
+    _need_cuda(ab_save, u, s_NM)
+    N, M = s_NM.shape
+    H = u.shape[1]
+    _call("momoe_swiglu_bwd_saved", _ptr(ab_save), _ptr(u), _ptr(s_NM), s_NM.stride(0),
+                                       s_NM.stride(1), _ptr(idx), _ptr(cumsums), Msave, _ptr(gz),
+                                       _ptr(hs), _ptr(gs_part), gs_part.shape[0], M, H, N,
+                                       idx.numel(), _stream())
 
 
 def gs_scatter(gs_part, idx, cumsums, Gs_NM):

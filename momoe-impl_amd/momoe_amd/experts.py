@@ -100,15 +100,20 @@ class MoEFunction(torch.autograd.Function):
         with torch.cuda.device(dev):
             Gy = G_y_BSD.reshape(M, D).to(device=dev, dtype=torch.bfloat16).contiguous()
 
-            # a|b for the rows that were not saved are recomputed straight into the buffer
-            # that the next kernel turns, in place, into [G_a|G_b].
+            # dL/dh before the gate weight, in sorted order
+            u = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
+            _hip.dgrad_h(Gy, W2, idx, table, u)
+            # SwiGLU backward: rows with saved a|b read them; the others recompute a|b = x.Wl1
+            # and consume them straight from the GEMM's accumulators
             gz = torch.empty((msum, 2 * H), device=dev, dtype=torch.bfloat16)
-            if msave < msum:
-                _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, None, gz, msave, msum)
             hs = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
             nparts = (H + _hip.GS_BLOCK - 1) // _hip.GS_BLOCK
             gs_part = torch.empty((nparts, msum), device=dev, dtype=torch.float32)
-            _hip.dgrad_h_swiglu_bwd(Gy, W2, s, idx, table, ab_save, msave, gz, hs, gs_part)
+            if msave > 0:
+                _hip.swiglu_bwd_saved(ab_save, u, s, idx, cumsums, msave, gz, hs, gs_part)
+            if msave < msum:
+                _hip.lin1_swiglu_bwd(x_MD, W1, idx, table, u, s, msave, gz, hs, gs_part)
+            del u
 
             G_s = None
             if need_s:
