@@ -146,6 +146,8 @@ struct RDma {
 #pragma unroll
     for (int j = 0; j < NCH; ++j) dma16(b, off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
   }
+  template <int S>
+  __device__ __forceinline__ void issue_head(uint32_t stage) { issue(S, stage); }
   // 32 rows starting at r0 (multiple of 32), k-step kk (16 k-values)
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int r0, int kk) {
     const int l = threadIdx.x & 63;
@@ -157,19 +159,22 @@ struct RDma {
 
 // ---- k-strided operand, 256 columns -----------------------------------------------------
 // LDS stage: k-row k at elements [256k, 256k+256); 16-byte piece p of the row is stored
-// at position p ^ (2*(k&3)), so the 4 k-rows x 32 bytes that a 16-lane group of the
-// transpose read touches fall into 4 different bank quarters.  A deposit covers two k-rows
-// (lanes 0-31 / 32-63); wave w deposits k-rows [4w, 4w+4).
+// at position p ^ swz(k), swz(k) = 4*(k&3) + 16*((k>>3)&1): the 8 k-rows x 64 bytes that one
+// transpose read of a wave touches then fall into 8 different 64-byte bank groups (measured
+// 124 B/clk against 113 for a swizzle that only separates the 4 k-rows of a 16-lane group;
+// the instruction tops out at 128).  A deposit covers two k-rows (lanes 0-31 / 32-63); wave w
+// deposits k-rows [4w, 4w+4).
 struct TLayout {
   static constexpr int COLS = 256;
   static constexpr int NCH = kBK / (2 * kWaves);  // deposits per wave per stage
   static constexpr int LDS_ELEMS = kBK * COLS;
+  static __device__ __forceinline__ int swz(int krow) { return 4 * (krow & 3) + 16 * ((krow >> 3) & 1); }
 
   // k-row and logical column (multiple of 8) fetched by this lane in deposit j
   static __device__ __forceinline__ void lane_piece(int j, int& krow, int& col) {
     const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
     krow = w * (2 * NCH) + j * 2 + (l >> 5);
-    col = ((l & 31) ^ (2 * (krow & 3))) * 8;
+    col = ((l & 31) ^ swz(krow)) * 8;
   }
   static __device__ __forceinline__ uint32_t deposit(uint32_t stage, int j) {
     return stage + ((threadIdx.x >> 6) * NCH + j) * (kChunkElems * 2);
@@ -179,7 +184,8 @@ struct TLayout {
     const int l = threadIdx.x & 63;
     const int krow = kk * 16 + 8 * (l >> 5) + ((l & 15) >> 2);
     const int col = c0 + 16 * ((l & 31) >> 4) + 4 * (l & 3);
-    const bf16* p = stage + krow * COLS + (((col >> 3) ^ (2 * (krow & 3))) << 3) + (col & 7);
+    // k-rows krow and krow+4 share the swizzle, so the second read is a fixed distance away
+    const bf16* p = stage + krow * COLS + (((col >> 3) ^ swz(krow)) << 3) + (col & 7);
     const bf16x4 lo = lds_read_tr4(p);
     const bf16x4 hi = lds_read_tr4(p + 4 * COLS);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -214,6 +220,8 @@ struct TDma {
 #pragma unroll
     for (int j = 0; j < NCH; ++j) dma16(b, off[j], L::deposit(stage, j));
   }
+  template <int S>
+  __device__ __forceinline__ void issue_head(uint32_t stage) { issue(S, stage); }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
     return L::frag(stage, c0, kk);
   }
@@ -221,8 +229,9 @@ struct TDma {
 
 // k-strided operand whose k-rows are the sorted rows [row_begin,row_end) of one expert,
 // optionally gathered through an index; k-rows past row_end read the zero block.  The row
-// ids of a deposit are a wave-uniform pair: they are fetched with scalar loads one stage
-// ahead of their use.
+// ids of a deposit are a wave-uniform pair, fetched with scalar loads: those of the first
+// kFirst stages once per expert (every tile of the expert starts with the same rows), the
+// later ones one stage ahead of their use.
 struct TGatherDma {
   using L = TLayout;
   static constexpr int NCH = L::NCH;
@@ -232,49 +241,66 @@ struct TGatherDma {
   const int32_t* gather;
   int row_begin, row_end;
   int col[NCH];
-  int32_t id0[NCH], id1[NCH];
+  struct Ids {
+    int32_t a[NCH], b[NCH];  // row ids of the two k-rows of each deposit, -1 = past the end
+  };
+  Ids head0, head1, head2;  // this wave's k-rows in the first three stages
+  Ids ids;                  // for the next issue() call
+  static_assert(kFirst == 3, "three cached stages");
 
-  __device__ __forceinline__ void fetch_rows(int kt) {
+  __device__ __forceinline__ Ids row_pairs(int kt) const {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    Ids out;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       const int rr = row_begin + kt * kBK + w * (2 * NCH) + j * 2;
-      int32_t a = -1, b = -1;
-      if (rr < row_end) a = gather ? load_uniform(gather + rr) : rr;
-      if (rr + 1 < row_end) b = gather ? load_uniform(gather + rr + 1) : rr + 1;
-      id0[j] = a;
-      id1[j] = b;
+      out.a[j] = -1;
+      out.b[j] = -1;
+      if (rr < row_end) out.a[j] = gather ? load_uniform(gather + rr) : rr;
+      if (rr + 1 < row_end) out.b[j] = gather ? load_uniform(gather + rr + 1) : rr + 1;
     }
+    return out;
   }
-  // columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
-  __device__ __forceinline__ void init(const bf16* mat_, int64_t ld_, const int32_t* gather_,
-                                       int col0, int ncols, int rb, int re) {
-    mat = mat_;
-    ld = ld_;
+  // once per expert
+  __device__ __forceinline__ void set_rows(const int32_t* gather_, int rb, int re) {
     gather = gather_;
     row_begin = rb;
     row_end = re;
+    head0 = row_pairs(0);
+    head1 = row_pairs(1);
+    head2 = row_pairs(2);
+  }
+  // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
+  __device__ __forceinline__ void set_cols(const bf16* mat_, int64_t ld_, int col0, int ncols) {
+    mat = mat_;
+    ld = ld_;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       int krow, c;
       L::lane_piece(j, krow, c);
       col[j] = col0 + c < ncols ? col0 + c : 0;
     }
-    fetch_rows(0);
   }
-  // must be called with kt = 0, 1, 2, ... in order: uses the row ids fetched for kt and
-  // starts fetching those of kt+1
-  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+  __device__ __forceinline__ void deposit(const Ids v, uint32_t stage) const {
     const bool upper = (threadIdx.x & 63) >= 32;
-    const bf16* src[NCH];
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int32_t id = upper ? id1[j] : id0[j];
-      src[j] = id >= 0 ? mat + (int64_t)id * ld + col[j] : zero_chunk();
+      const int32_t id = upper ? v.b[j] : v.a[j];
+      dma16(id >= 0 ? mat + (int64_t)id * ld + col[j] : zero_chunk(), L::deposit(stage, j));
     }
-    fetch_rows(kt + 1);
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) dma16(src[j], L::deposit(stage, j));
+  }
+  // stage S < kFirst of a tile; the last of them starts the fetch for issue(kFirst)
+  template <int S>
+  __device__ __forceinline__ void issue_head(uint32_t stage) {
+    deposit(S == 0 ? head0 : S == 1 ? head1 : head2, stage);
+    if (S == kFirst - 1) ids = row_pairs(kFirst);
+  }
+  // must be called with kt = kFirst, kFirst+1, ... in order: uses the row ids fetched for kt
+  // and starts fetching those of kt+1
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+    const Ids cur = ids;
+    ids = row_pairs(kt + 1);
+    deposit(cur, stage);
   }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
     return L::frag(stage, c0, kk);
@@ -309,24 +335,53 @@ __device__ __forceinline__ void gemm_issue(AOp& A, BOp& B, StageRing<AOp, BOp>& 
   B.issue(kt, st + AOp::LDS_ELEMS * 2);
 }
 
-// Request the first three stages of a tile.  May be called right after the previous tile's
-// main loop, while other waves still multiply its last stage: the other three buffers were
+// Request the first kFirst stages of a tile.  May be called right after the previous tile's
+// main loop, while other waves still multiply its last stage: the other buffers were
 // released by that tile's last barrier.
+template <int S, class AOp, class BOp>
+__device__ __forceinline__ void gemm_issue_head(AOp& A, BOp& B, StageRing<AOp, BOp>& ring) {
+  const uint32_t st = ring.buf_addr(S);
+  A.template issue_head<S>(st);
+  B.template issue_head<S>(st + AOp::LDS_ELEMS * 2);
+}
 template <class AOp, class BOp>
 __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp>& ring,
                                                  int ktiles) {
-  gemm_issue(A, B, ring, 0);
-#pragma unroll
-  for (int s = 1; s < kFirst; ++s)
-    if (ktiles > s) gemm_issue(A, B, ring, s);
+  static_assert(kFirst == 3, "written for three stages ahead");
+  gemm_issue_head<0>(A, B, ring);
+  if (ktiles > 1) gemm_issue_head<1>(A, B, ring);
+  if (ktiles > 2) gemm_issue_head<2>(A, B, ring);
 }
 
-// wait until the deposits of stage kt have landed, when the stages up to kt+kStages-2 have
-// been requested and everything older than stage kt is known to be complete
-template <int LOADS>
+// Vector-memory operations of a wave complete in the order they were issued (loads and stores
+// share the one counter on this architecture), so "at most n outstanding" means "all but the
+// youngest n are done".  The waits below allow exactly the operations known to be younger than
+// the stage that is needed.  PENDING is a lower bound on the number of stores the wave issued
+// between requesting the first kFirst stages of this tile and entering its main loop (the
+// previous tile's epilogue): those sit between stage kFirst-1 and stage kFirst in the queue and
+// may stay in flight while the first stages are multiplied, instead of being drained first.
+template <int LOADS, int PENDING>
+__device__ __forceinline__ void wait_first_stage(int ktiles) {
+  static_assert((kFirst - 1) * LOADS + PENDING <= 63, "vmcnt is a 6-bit counter");
+  static_assert(kFirst == 3 || kFirst == 4, "wait ladder written for 3 or 4 stages ahead");
+  if (kFirst == 4 && ktiles > 3) wait_vmcnt<3 * LOADS + PENDING>();
+  else if (ktiles > 2) wait_vmcnt<2 * LOADS + PENDING>();
+  else if (ktiles > 1) wait_vmcnt<LOADS + PENDING>();
+  else wait_vmcnt<PENDING>();
+}
+// wait until the deposits of stage kt (>= 1) have landed, when the stages up to kt+kStages-2
+// have been requested and everything older than stage kt is known to be complete
+template <int LOADS, int PENDING>
 __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
-  static_assert((kStages - 2) * LOADS <= 63, "vmcnt is a 6-bit counter");
+  static_assert((kStages - 2) * LOADS + PENDING <= 63, "vmcnt is a 6-bit counter");
   static_assert(kStages == 4 || kStages == 5, "wait ladder written for 4 or 5 stages");
+  if (PENDING > 0 && kt < kFirst) {
+    if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS + PENDING>();
+    else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS + PENDING>();
+    else if (kt + 1 < ktiles) wait_vmcnt<LOADS + PENDING>();
+    else wait_vmcnt<PENDING>();
+    return;
+  }
   if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS>();
   else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
   else if (kt + 1 < ktiles) wait_vmcnt<LOADS>();
@@ -341,7 +396,7 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
 // under the whole main loop (they enter the vmcnt queue between two stages, which can only
 // make the stage waits err on the long side).  On return the ring has advanced to the next
 // tile; all buffers but the last stage's are free, other waves may still be reading that one.
-template <class AOp, class BOp, int FM, int FN, int NA, class Hook>
+template <class AOp, class BOp, int FM, int FN, int NA, int PENDING, class Hook>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                               StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
                                               const int (&n_org)[FN], Hook hook) {
@@ -367,9 +422,9 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   // The scheduling fences keep the compiler from hoisting fragment reads across k-steps.
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
-  // Everything requested so far has landed (this also drains the previous tile's stores);
-  // every wave is done reading the previous tile, whose last buffer the next stage will reuse.
-  wait_vmcnt<0>();
+  // Stage 0 has landed; every wave is done reading the previous tile, whose last buffer the
+  // next stage will reuse.
+  wait_first_stage<LOADS, PENDING>(ktiles);
   wait_lgkm0();
   __builtin_amdgcn_s_barrier();
   fence();
@@ -388,7 +443,7 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
     fence();
     // stage kt+1 has landed; all LDS reads of stage kt have returned, so its buffer may be
     // overwritten once every wave is past the barrier
-    wait_stage<LOADS>(kt + 1, ktiles);
+    wait_stage<LOADS, PENDING>(kt + 1, ktiles);
     wait_lgkm0();
     __builtin_amdgcn_s_barrier();
     fence();
@@ -407,18 +462,25 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
 }
 
 // main loop for a wave that owns rows [m_org[0], m_org[0] + 32*FM) of a tile whose first
-// `rows` rows are valid
-template <class AOp, class BOp, int FM, int FN, class Hook>
+// `rows` rows are valid.  `stores_pending`: the wave issued at least PENDING stores since the
+// first stages of this tile were requested (see wait_first_stage).
+template <class AOp, class BOp, int FM, int FN, int PENDING, class Hook>
 __device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                           StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                          const int (&n_org)[FN], int rows, Hook hook) {
+                                          const int (&n_org)[FN], int rows, bool stores_pending,
+                                          Hook hook) {
   static_assert(FM == 4, "dispatch written for 4 fragment rows per wave");
   const int na = __builtin_amdgcn_readfirstlane(min(FM, max(0, (rows - m_org[0] + 31) >> 5)));
-  if (na == 4) gemm_mainloop<AOp, BOp, FM, FN, 4>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else gemm_mainloop<AOp, BOp, FM, FN, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  if (na == 4) {
+    if (PENDING > 0 && stores_pending)
+      gemm_mainloop<AOp, BOp, FM, FN, 4, PENDING>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+    else
+      gemm_mainloop<AOp, BOp, FM, FN, 4, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  }
+  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else gemm_mainloop<AOp, BOp, FM, FN, 0, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
 }
 
 // the workgroup's dynamic LDS (size given at launch)
@@ -498,7 +560,7 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
     TileSched::Raw rn;
-    gemm_rows<AOp, BOp, FM, FN>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.rows, [&] {
+    gemm_rows<AOp, BOp, FM, FN, 0>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.rows, false, [&] {
       prog.late(c0, p0);
       if (c1.valid) prog.gather(c1, p1);
       rn = sched.fetch();

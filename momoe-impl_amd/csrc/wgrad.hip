@@ -28,9 +28,11 @@ struct WgradArgs {
 };
 
 struct WTile {
-  int expert, x0, y0, rb, re;
+  int expert, x0, y0;
   bool valid;
 };
+
+constexpr int kTileStores = FM * RowStager<2>::PASSES;  // stores per lane in a full tile's epilogue
 
 // Persistent workgroups.  id%8 is the XCD a workgroup lands on; experts are dealt
 // round-robin to the XCDs and every tile of an expert runs on that one XCD, so the
@@ -51,19 +53,27 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
       t.expert = expert;
       t.x0 = (q / p.tiles_y) * BX;
       t.y0 = (q % p.tiles_y) * BY;
-      t.rb = load_uniform(p.cumsums + expert);
-      t.re = load_uniform(p.cumsums + expert + 1);
       t.valid = true;
       break;
     }
     return t;
   };
   TGatherDma A, B;
+  int cur_expert = -1, rb = 0, re = 0;
+  // the rows of an expert (and the ids of the first of them) are looked up when the
+  // workgroup moves on to a new expert; every tile of the expert then reuses them
   auto start = [&](const WTile& t) {
-    if (t.re <= t.rb) return;  // expert without rows: nothing to load, zeros are stored
-    A.init(p.a, p.lda, p.ga, t.x0, p.X, t.rb, t.re);
-    B.init(p.b, p.ldb, p.gb, t.y0, p.Y, t.rb, t.re);
-    gemm_issue_first(A, B, ring, (t.re - t.rb + kBK - 1) / kBK);
+    if (t.expert != cur_expert) {
+      cur_expert = t.expert;
+      rb = load_uniform(p.cumsums + t.expert);
+      re = load_uniform(p.cumsums + t.expert + 1);
+      A.set_rows(p.ga, rb, re);
+      B.set_rows(p.gb, rb, re);
+    }
+    if (re <= rb) return;  // expert without rows: nothing to load, zeros are stored
+    A.set_cols(p.a, p.lda, t.x0, p.X);
+    B.set_cols(p.b, p.ldb, t.y0, p.Y);
+    gemm_issue_first(A, B, ring, (re - rb + kBK - 1) / kBK);
   };
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
   const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
@@ -73,13 +83,18 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
   WTile tc = next_tile();
   if (!tc.valid) return;
   start(tc);
+  bool stores_pending = false;  // a full tile's worth of stores was issued after start()
   while (true) {
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
-    const int ktiles = (tc.re - tc.rb + kBK - 1) / kBK;
-    if (ktiles > 0)
-      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
+    const int ktiles = (re - rb + kBK - 1) / kBK;  // rows of tc's expert (start(tc) ran last)
     const WTile nx = next_tile();
+    if (ktiles > 0) {
+      if (stores_pending)
+        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, kTileStores>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
+      else
+        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, 0>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
+    }
     if (nx.valid) start(nx);
 
     bf16* out = p.gw + (int64_t)tc.expert * p.X * p.Y;
@@ -98,6 +113,8 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
         return out + (int64_t)x * p.Y + y0 + col;
       });
     }
+    // every lane stored in every pass iff the tile lies fully inside the matrix
+    stores_pending = tc.x0 + BX <= p.X && tc.y0 + BY <= p.Y;
     if (!nx.valid) break;
     tc = nx;
   }
