@@ -228,42 +228,45 @@ struct TDma {
 };
 
 // k-strided operand whose k-rows are the sorted rows [row_begin,row_end) of one expert,
-// optionally gathered through an index; k-rows past row_end read the zero block.  The row
-// ids of a deposit are a wave-uniform pair, fetched with scalar loads: those of the first
-// kFirst stages once per expert (every tile of the expert starts with the same rows), the
-// later ones one stage ahead of their use.
+// optionally gathered through an index.  k-rows past row_end are pointed at the expert's last
+// row (any readable row would do): the main loop zeroes the M-side fragments of those k-values
+// in the last stage, so they add nothing.  The row ids of a deposit are a wave-uniform pair,
+// fetched with scalar loads: those of the first kFirst stages once per expert (every tile of
+// the expert starts with the same rows), the later ones one stage ahead of their use.  Sources
+// are given as the matrix base plus a 32-bit byte offset per lane (the form with a full
+// 64-bit address per lane costs ~20% of the whole GEMM), so a matrix must stay below 4 GiB.
 struct TGatherDma {
   using L = TLayout;
   static constexpr int NCH = L::NCH;
   static constexpr int LDS_ELEMS = L::LDS_ELEMS;
-  const bf16* mat;
-  int64_t ld;
+  const bf16* mat;  // wave-uniform
+  uint32_t ldb;     // bytes between rows
   const int32_t* gather;
   int row_begin, row_end;
-  int col[NCH];
-  struct Ids {
-    int32_t a[NCH], b[NCH];  // row ids of the two k-rows of each deposit, -1 = past the end
+  uint32_t colb[NCH];  // byte offset of this lane's columns in deposit j
+  struct Offs {
+    uint32_t a[NCH], b[NCH];  // byte offsets of the two k-rows of each deposit
   };
-  Ids head0, head1, head2;  // this wave's k-rows in the first three stages
-  Ids ids;                  // for the next issue() call
+  Offs head0, head1, head2;  // this wave's k-rows in the first three stages
+  Offs next;                 // for the next issue() call
   static_assert(kFirst == 3, "three cached stages");
 
-  __device__ __forceinline__ Ids row_pairs(int kt) const {
+  __device__ __forceinline__ Offs row_pairs(int kt) const {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    Ids out;
+    Offs out;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int rr = row_begin + kt * kBK + w * (2 * NCH) + j * 2;
-      out.a[j] = -1;
-      out.b[j] = -1;
-      if (rr < row_end) out.a[j] = gather ? load_uniform(gather + rr) : rr;
-      if (rr + 1 < row_end) out.b[j] = gather ? load_uniform(gather + rr + 1) : rr + 1;
+      const int ra = min(row_begin + kt * kBK + w * (2 * NCH) + j * 2, row_end - 1);
+      const int rb = min(ra + 1, row_end - 1);
+      out.a[j] = (uint32_t)(gather ? load_uniform(gather + ra) : ra) * ldb;
+      out.b[j] = (uint32_t)(gather ? load_uniform(gather + rb) : rb) * ldb;
     }
     return out;
   }
-  // once per expert
-  __device__ __forceinline__ void set_rows(const int32_t* gather_, int rb, int re) {
+  // once per expert (re > rb); ld_ = elements between rows of the matrix
+  __device__ __forceinline__ void set_rows(const int32_t* gather_, int64_t ld_, int rb, int re) {
     gather = gather_;
+    ldb = (uint32_t)(ld_ * 2);
     row_begin = rb;
     row_end = re;
     head0 = row_pairs(0);
@@ -271,35 +274,32 @@ struct TGatherDma {
     head2 = row_pairs(2);
   }
   // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
-  __device__ __forceinline__ void set_cols(const bf16* mat_, int64_t ld_, int col0, int ncols) {
+  __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
     mat = mat_;
-    ld = ld_;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       int krow, c;
       L::lane_piece(j, krow, c);
-      col[j] = col0 + c < ncols ? col0 + c : 0;
+      colb[j] = (uint32_t)(col0 + c < ncols ? col0 + c : 0) * 2;
     }
   }
-  __device__ __forceinline__ void deposit(const Ids v, uint32_t stage) const {
+  __device__ __forceinline__ void deposit(const Offs v, uint32_t stage) const {
     const bool upper = (threadIdx.x & 63) >= 32;
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int32_t id = upper ? v.b[j] : v.a[j];
-      dma16(id >= 0 ? mat + (int64_t)id * ld + col[j] : zero_chunk(), L::deposit(stage, j));
-    }
+    for (int j = 0; j < NCH; ++j)
+      dma16(mat, (upper ? v.b[j] : v.a[j]) + colb[j], L::deposit(stage, j));
   }
   // stage S < kFirst of a tile; the last of them starts the fetch for issue(kFirst)
   template <int S>
   __device__ __forceinline__ void issue_head(uint32_t stage) {
     deposit(S == 0 ? head0 : S == 1 ? head1 : head2, stage);
-    if (S == kFirst - 1) ids = row_pairs(kFirst);
+    if (S == kFirst - 1) next = row_pairs(kFirst);
   }
-  // must be called with kt = kFirst, kFirst+1, ... in order: uses the row ids fetched for kt
+  // must be called with kt = kFirst, kFirst+1, ... in order: uses the offsets fetched for kt
   // and starts fetching those of kt+1
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
-    const Ids cur = ids;
-    ids = row_pairs(kt + 1);
+    const Offs cur = next;
+    next = row_pairs(kt + 1);
     deposit(cur, stage);
   }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
@@ -392,6 +392,7 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
 // stages must already have been requested with gemm_issue_first.  NA is the number of 32-row
 // fragment rows of this wave that hold valid rows (wave-uniform): the others are neither read
 // nor multiplied; with NA = 0 the wave only takes part in the transfers and barriers.
+// `ktail` (1..kBK) is the number of k-values of the last stage that exist.
 // `hook` runs once, right after the barrier that opens the tile: loads issued there travel
 // under the whole main loop (they enter the vmcnt queue between two stages, which can only
 // make the stage waits err on the long side).  On return the ring has advanced to the next
@@ -399,7 +400,7 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
 template <class AOp, class BOp, int FM, int FN, int NA, int PENDING, class Hook>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                               StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                              const int (&n_org)[FN], Hook hook) {
+                                              const int (&n_org)[FN], Hook hook, int ktail = kBK) {
   static_assert(kKSteps == 2, "written for 2 k-steps per stage");
   static_assert(NA >= 0 && NA <= FM, "active fragment rows");
   constexpr int LOADS = AOp::NCH + BOp::NCH;
@@ -454,6 +455,23 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
     fence();
   }
   load_frags(ktiles - 1, 1);
+  if (ktail < kBK) {
+    // only the first `ktail` k-values of the last stage exist: zero the rest on the M side
+    // (a lane holds k-values 16*kk + 8*(lane/32) + 0..7 of its row, two per register)
+    wait_lgkm0();
+#pragma unroll
+    for (int kk = 0; kk < kKSteps; ++kk) {
+      const int nvalid = ktail - 16 * kk - 8 * (int)((threadIdx.x & 63) >> 5);
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        u32x4 v = __builtin_bit_cast(u32x4, af[kk][i]);
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          v[d] &= nvalid >= 2 * d + 2 ? 0xFFFFFFFFu : nvalid == 2 * d + 1 ? 0x0000FFFFu : 0u;
+        af[kk][i] = __builtin_bit_cast(bf16x8, v);
+      }
+    }
+  }
   multiply(0);
   fence();
   multiply(1);

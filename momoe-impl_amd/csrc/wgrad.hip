@@ -1,8 +1,8 @@
 // Weight-gradient grouped GEMM: GW[i] = A_i^T . B_i, contracting over the sorted
 // rows of expert i.  Both operands are stored [row][feature], i.e. k-strided, so
 // both go through the LDS transpose read.  Rows may be gathered through an index
-// (x and G_y are never materialised in sorted order); rows past the expert's last
-// one read a block of zeros.
+// (x and G_y are never materialised in sorted order); the k-values past the expert's
+// last row are zeroed in registers.
 #include "gemm_tile.hpp"
 
 namespace momoe {
@@ -67,12 +67,14 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
       cur_expert = t.expert;
       rb = load_uniform(p.cumsums + t.expert);
       re = load_uniform(p.cumsums + t.expert + 1);
-      A.set_rows(p.ga, rb, re);
-      B.set_rows(p.gb, rb, re);
+      if (re > rb) {
+        A.set_rows(p.ga, p.lda, rb, re);
+        B.set_rows(p.gb, p.ldb, rb, re);
+      }
     }
     if (re <= rb) return;  // expert without rows: nothing to load, zeros are stored
-    A.set_cols(p.a, p.lda, t.x0, p.X);
-    B.set_cols(p.b, p.ldb, t.y0, p.Y);
+    A.set_cols(p.a, t.x0, p.X);
+    B.set_cols(p.b, t.y0, p.Y);
     gemm_issue_first(A, B, ring, (re - rb + kBK - 1) / kBK);
   };
   const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
@@ -88,12 +90,13 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
     const int ktiles = (re - rb + kBK - 1) / kBK;  // rows of tc's expert (start(tc) ran last)
+    const int ktail = re - rb - (ktiles - 1) * kBK;
     const WTile nx = next_tile();
     if (ktiles > 0) {
       if (stores_pending)
-        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, kTileStores>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
+        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, kTileStores>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
       else
-        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, 0>(A, B, acc, ktiles, ring, m_org, n_org, [] {});
+        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, 0>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
     }
     if (nx.valid) start(nx);
 
@@ -135,6 +138,9 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
   if (((uintptr_t)A_rows & 15) || ((uintptr_t)B_rows & 15) || ((uintptr_t)GW_NXY & 7))
     return MOMOE_ERR_BAD_ARG;
   if (Msum >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
+  // rows are addressed with 32-bit byte offsets from the matrix base (a gathered matrix has at
+  // most Msum rows: every row id is a token that holds at least one pair)
+  if (Msum * lda * 2 >= (1ll << 32) || Msum * ldb * 2 >= (1ll << 32)) return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
   if (cdiv64(N, 8) * tiles_x * tiles_y >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
