@@ -151,15 +151,16 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
 /* momoe_wgrad replaces weights_update_kernel (momoe/momoe.py:356-412):
  *   GW[i][x][y] = bf16( sum over sorted rows r of expert i of A[ra(r)][x] * B[rb(r)][y] )
  * with ra(r) = a_gather ? a_gather[r] : r (same for rb).  A bf16 with row stride lda
- * (>= X), B bf16 with row stride ldb (>= Y); both must span less than 4 GiB
- * (Msum * ld * 2 bytes).  Experts without rows get exact zeros.
+ * (>= X), B bf16 with row stride ldb (>= Y).  M = number of tokens (rows of a gathered
+ * matrix, and the most rows an expert can hold); M * ld * 2 bytes must stay below 4 GiB.
+ * Experts without rows get exact zeros.
  * Wl2 gradient: A = hs (X=H), B = G_y gathered by idx (Y=D).
  * Wl1 gradient: A = x gathered by idx (X=D), B = gz (Y=2H).
  */
 int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
                 const void* B_rows, int64_t ldb, const int32_t* b_gather,
                 const int32_t* cumsums_N1, void* GW_NXY,
-                int64_t N, int64_t X, int64_t Y, int64_t Msum, void* stream);
+                int64_t M, int64_t N, int64_t X, int64_t Y, int64_t Msum, void* stream);
 
 /* ---- router ----------------------------------------------------------------
  * momoe_router_fwd replaces the elementwise part of TopKRouterFunction.forward

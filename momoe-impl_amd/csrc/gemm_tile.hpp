@@ -233,8 +233,10 @@ struct TDma {
 // in the last stage, so they add nothing.  The row ids of a deposit are a wave-uniform pair,
 // fetched with scalar loads: those of the first kFirst stages once per expert (every tile of
 // the expert starts with the same rows), the later ones one stage ahead of their use.  Sources
-// are given as the matrix base plus a 32-bit byte offset per lane (the form with a full
-// 64-bit address per lane costs ~20% of the whole GEMM), so a matrix must stay below 4 GiB.
+// are given as a wave-uniform base plus a 32-bit byte offset per lane (the form with a full
+// 64-bit address per lane costs ~20% of the whole GEMM): the base is the matrix for a
+// gathered operand and the expert's first row otherwise, so (number of tokens) x (row pitch)
+// must stay below 4 GiB.
 struct TGatherDma {
   using L = TLayout;
   static constexpr int NCH = L::NCH;
@@ -258,8 +260,8 @@ struct TGatherDma {
     for (int j = 0; j < NCH; ++j) {
       const int ra = min(row_begin + kt * kBK + w * (2 * NCH) + j * 2, row_end - 1);
       const int rb = min(ra + 1, row_end - 1);
-      out.a[j] = (uint32_t)(gather ? load_uniform(gather + ra) : ra) * ldb;
-      out.b[j] = (uint32_t)(gather ? load_uniform(gather + rb) : rb) * ldb;
+      out.a[j] = (uint32_t)(gather ? load_uniform(gather + ra) : ra - row_begin) * ldb;
+      out.b[j] = (uint32_t)(gather ? load_uniform(gather + rb) : rb - row_begin) * ldb;
     }
     return out;
   }
@@ -275,7 +277,7 @@ struct TGatherDma {
   }
   // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
   __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
-    mat = mat_;
+    mat = gather ? mat_ : (const bf16*)((const char*)mat_ + (int64_t)row_begin * ldb);
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
       int krow, c;

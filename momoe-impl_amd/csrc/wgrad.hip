@@ -130,17 +130,18 @@ using namespace momoe;
 
 extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
                            const void* B_rows, int64_t ldb, const int32_t* b_gather,
-                           const int32_t* cumsums_N1, void* GW_NXY, int64_t N, int64_t X,
-                           int64_t Y, int64_t Msum, void* stream) {
+                           const int32_t* cumsums_N1, void* GW_NXY, int64_t M, int64_t N,
+                           int64_t X, int64_t Y, int64_t Msum, void* stream) {
   if (!A_rows || !B_rows || !cumsums_N1 || !GW_NXY) return MOMOE_ERR_BAD_ARG;
-  if (N <= 0 || X <= 0 || Y <= 0 || Msum <= 0 || lda < X || ldb < Y) return MOMOE_ERR_BAD_ARG;
+  if (M <= 0 || N <= 0 || X <= 0 || Y <= 0 || Msum <= 0 || lda < X || ldb < Y)
+    return MOMOE_ERR_BAD_ARG;
   if (X % 8 != 0 || Y % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return MOMOE_ERR_UNSUPPORTED;
   if (((uintptr_t)A_rows & 15) || ((uintptr_t)B_rows & 15) || ((uintptr_t)GW_NXY & 7))
     return MOMOE_ERR_BAD_ARG;
   if (Msum >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
-  // rows are addressed with 32-bit byte offsets from the matrix base (a gathered matrix has at
-  // most Msum rows: every row id is a token that holds at least one pair)
-  if (Msum * lda * 2 >= (1ll << 32) || Msum * ldb * 2 >= (1ll << 32)) return MOMOE_ERR_UNSUPPORTED;
+  // rows are addressed with 32-bit byte offsets from the matrix base (gathered: M rows) or from
+  // the expert's first row (an expert holds a token at most once: at most M rows)
+  if (M * lda * 2 >= (1ll << 32) || M * ldb * 2 >= (1ll << 32)) return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
   if (cdiv64(N, 8) * tiles_x * tiles_y >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,

@@ -46,7 +46,7 @@ _SIGNATURES = {
                                       _i64, _i64, _i64, _i64, _p]),
     "momoe_gs_scatter": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _p]),
     "momoe_dgrad_x": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
-    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "momoe_router_fwd": (_int, [_p, _int, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p]),
     "momoe_router_bwd": (_int, [_p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p]),
 }
@@ -211,11 +211,11 @@ def dgrad_x(gz, Wl1_ND2H, table, gxs, M):
                               gz.shape[0], _stream())
 
 
-def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, Msum):
+def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, M, Msum):
     N, X, Y = GW_NXY.shape
     _call("momoe_wgrad", _ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
-                            B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), N, X, Y,
-                            Msum, _stream())
+                            B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X,
+                            Y, Msum, _stream())
 
 
 # ---------------------------------------------------------------- router

@@ -124,13 +124,13 @@ class MoEFunction(torch.autograd.Function):
             G_W2 = None
             if need_w2:
                 G_W2 = torch.empty_like(W2)
-                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, msum)
+                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, M, msum)
             del hs
 
             G_W1 = None
             if need_w1:
                 G_W1 = torch.empty_like(W1)
-                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, msum)
+                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, M, msum)
 
             G_x_BSD = None
             if need_x:

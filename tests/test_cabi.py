@@ -49,7 +49,7 @@ def test_size_queries_and_argument_validation(lib):
     # null pointers / bad sizes are rejected on the host before anything is launched
     z = ctypes.c_void_p(0)
     assert lib.momoe_combine(z, z, z, i64(1), i64(8), i64(1), i64(1), z) == 1
-    assert lib.momoe_wgrad(z, i64(8), z, z, i64(8), z, z, z, i64(1), i64(8), i64(8), i64(1), z) == 1
+    assert lib.momoe_wgrad(z, i64(8), z, z, i64(8), z, z, z, i64(1), i64(1), i64(8), i64(8), i64(1), z) == 1
 
 
 def test_host_modules_refuse_cpu_tensors():
