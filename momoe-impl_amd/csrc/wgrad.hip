@@ -34,27 +34,69 @@ struct WTile {
 
 constexpr int kTileStores = FM * RowStager<2>::PASSES;  // stores per lane in a full tile's epilogue
 
-// Persistent workgroups.  id%8 is the XCD a workgroup lands on; experts are dealt
-// round-robin to the XCDs and every tile of an expert runs on that one XCD, so the
-// expert's rows are fetched from HBM once and re-read from that XCD's L2.
+constexpr int kEpilogueCost = 4;  // a tile's epilogue, in units of one k-stage of its main loop
+
+// Persistent workgroups.  id%8 is the XCD a workgroup lands on.  Tiles are numbered expert
+// by expert and cut into 8 contiguous runs of equal estimated cost (a tile costs its expert's
+// k-stages plus the epilogue), one per XCD: an expert's rows are then fetched from HBM by one
+// L2 (two for an expert that straddles a cut) and re-read from there by all of its tiles, and
+// an expert that holds far more rows than the others does not hold up one XCD.
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
   Ring ring(dyn_lds());
   const int tpe = p.tiles_x * p.tiles_y;
   const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
-  const int total = ((p.N + 7) >> 3) * tpe;  // tile slots of one XCD
-  int pos = blockIdx.x >> 3;
+
+  // pre[e] = cost of all tiles of the experts before e (exclusive prefix sum), in the stage ring
+  int64_t* pre = (int64_t*)dyn_lds();
+  int64_t* wave_tot = pre + p.N + 1;
+  {
+    const int per = (p.N + kThreads - 1) / kThreads;  // experts per thread, contiguous
+    const int e0 = min((int)threadIdx.x * per, p.N), e1 = min(e0 + per, p.N);
+    int64_t mine = 0;
+    for (int e = e0; e < e1; ++e)
+      mine += (int64_t)tpe * ((p.cumsums[e + 1] - p.cumsums[e] + kBK - 1) / kBK + kEpilogueCost);
+    int64_t incl = mine;  // inclusive scan over the wave, then over the waves
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int64_t v = __shfl_up(incl, o);
+      if ((int)(threadIdx.x & 63) >= o) incl += v;
+    }
+    if ((threadIdx.x & 63) == 63) wave_tot[threadIdx.x >> 6] = incl;
+    __syncthreads();
+    int64_t base = 0;
+    for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) base += wave_tot[w];
+    int64_t run = base + incl - mine;
+    for (int e = e0; e < e1; ++e) {
+      pre[e] = run;
+      run += (int64_t)tpe * ((p.cumsums[e + 1] - p.cumsums[e] + kBK - 1) / kBK + kEpilogueCost);
+    }
+    if (threadIdx.x == kThreads - 1) pre[p.N] = run;
+    __syncthreads();
+  }
+  // first tile whose cost interval starts at or after `c`
+  auto tile_at = [&](int64_t c) -> int64_t {
+    if (c >= pre[p.N]) return (int64_t)p.N * tpe;
+    int lo = 0, hi = p.N;  // pre[lo] <= c < pre[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (pre[mid] <= c) lo = mid; else hi = mid;
+    }
+    const int64_t each = (pre[lo + 1] - pre[lo]) / tpe;
+    return (int64_t)lo * tpe + (c - pre[lo] + each - 1) / each;
+  };
+  const int64_t total_cost = pre[p.N];
+  const int64_t g_begin = tile_at(total_cost * xcd / 8), g_end = tile_at(total_cost * (xcd + 1) / 8);
+  __syncthreads();  // the ring is handed to the transfers
+  int64_t pos = g_begin + (blockIdx.x >> 3);
   auto next_tile = [&]() {
     WTile t;
-    t.valid = false;
-    while (pos < total) {
-      const int expert = (pos / tpe) * 8 + xcd, q = pos % tpe;
+    t.valid = pos < g_end;
+    if (t.valid) {
+      const int expert = (int)(pos / tpe), q = (int)(pos % tpe);
       pos += stride;
-      if (expert >= p.N) continue;
       t.expert = expert;
       t.x0 = (q / p.tiles_y) * BX;
       t.y0 = (q % p.tiles_y) * BY;
-      t.valid = true;
-      break;
     }
     return t;
   };
@@ -143,7 +185,8 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
   // the expert's first row (an expert holds a token at most once: at most M rows)
   if (M * lda * 2 >= (1ll << 32) || M * ldb * 2 >= (1ll << 32)) return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
-  if (cdiv64(N, 8) * tiles_x * tiles_y >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  // the per-expert cost prefix sums live in LDS while the tiles are dealt out
+  if ((int64_t)tiles_x * tiles_y >= (1ll << 31) || N > 8192) return MOMOE_ERR_UNSUPPORTED;
   WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
               (bf16*)GW_NXY, (int)N, (int)X, (int)Y, tiles_x, tiles_y};
   static std::once_flag once;
