@@ -31,6 +31,8 @@ struct TileCoord {
   int row0;    // first sorted row of this tile
   int rows;    // valid rows in this tile (1..rows per tile)
   int tn;      // column block
+  int mbase;   // first tile row owned by this wave (waves 0-3 / 4-7 split the tile's rows)
+  int na;      // 32-row fragment rows owned by this wave (0..4)
   bool valid;
 };
 
@@ -83,13 +85,22 @@ struct TileSched {
     TileCoord tc;
     tc.valid = r.any;
     if (!r.any) return tc;
+    // The expert's rows are cut into its nt row tiles of equal height (a multiple of 32),
+    // not into full tiles plus a remainder: tiles that share a weight block then take equally
+    // long and stay in step, and no tile streams a whole weight block for a handful of rows.
     const int nt = (r.mi + bm - 1) / bm;
+    const int th = ((r.mi + nt - 1) / nt + 31) & ~31;
     const int qq = r.q - r.first * nb;
     const int tl = qq % nt;
     tc.tn = qq / nt;
     tc.expert = r.expert;
-    tc.row0 = r.rstart + tl * bm;
-    tc.rows = min(bm, r.mi - tl * bm);
+    tc.row0 = r.rstart + tl * th;
+    tc.rows = min(th, r.mi - tl * th);
+    // the tile's fragment rows are dealt to the two wave rows as evenly as possible
+    const int nf = (tc.rows + 31) >> 5, half = (nf + 1) >> 1;
+    const bool upper = threadIdx.x >= 256;
+    tc.mbase = upper ? 32 * half : 0;
+    tc.na = upper ? nf - half : half;
     return tc;
   }
   __device__ __forceinline__ TileCoord next() { return resolve(fetch()); }

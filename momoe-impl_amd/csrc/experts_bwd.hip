@@ -31,7 +31,6 @@ struct DhProg {
   };
   const DhArgs& p;
   const int ktiles, wn;
-  const int (&m_org)[FM];
   RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
@@ -51,7 +50,7 @@ struct DhProg {
     const int n0 = tc.tn * BN + wn * 64;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      if (m_org[i] >= tc.rows) break;
+      if (i >= tc.na) break;
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
@@ -59,7 +58,7 @@ struct DhProg {
           stager.put(f, q, pack_bf16x4(acc[f][i][4 * q], acc[f][i][4 * q + 1],
                                        acc[f][i][4 * q + 2], acc[f][i][4 * q + 3]));
       stager.flush([&](int row, int col) -> bf16* {
-        const int rl = m_org[i] + row;
+        const int rl = (tc.mbase + 32 * i) + row;
         if (rl >= tc.rows || n0 + col >= H) return nullptr;
         return p.u + ((int64_t)tc.row0 + rl) * H + n0 + col;
       });
@@ -70,11 +69,10 @@ struct DhProg {
 __global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.H + BN - 1) / BN);
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DhProg prog{p, p.D / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
+  DhProg prog{p, p.D / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
 }
 
 // SwiGLU backward for the sorted rows whose a|b were saved by the forward: one workgroup per
@@ -150,7 +148,6 @@ struct DxProg {
   struct Prep {};
   const DxArgs& p;
   const int ktiles, wn;
-  const int (&m_org)[FM];
   RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord&, Prep&) const {}
@@ -167,7 +164,7 @@ struct DxProg {
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      if (m_org[i] >= tc.rows) break;
+      if (i >= tc.na) break;
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
@@ -175,7 +172,7 @@ struct DxProg {
           stager.put(f, q, pack_bf16x4(acc[f][i][4 * q], acc[f][i][4 * q + 1],
                                        acc[f][i][4 * q + 2], acc[f][i][4 * q + 3]));
       stager.flush([&](int row, int col) -> bf16* {
-        const int rl = m_org[i] + row;
+        const int rl = (tc.mbase + 32 * i) + row;
         if (rl >= tc.rows || d0 + col >= D) return nullptr;
         return p.gxs + ((int64_t)tc.row0 + rl) * D + d0 + col;
       });
@@ -186,11 +183,10 @@ struct DxProg {
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DxProg prog{p, (2 * p.H) / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
+  DxProg prog{p, (2 * p.H) / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
 }
 
 __global__ __launch_bounds__(256) void gs_scatter_kernel(const float* __restrict__ part, int nparts,

@@ -48,7 +48,6 @@ struct Lin1Prog {
   };
   const Lin1Args& p;
   const int ktiles, wn;
-  const int (&m_org)[FM];
   bf16* epi;  // store staging; in the backward also the row-sum exchange
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
@@ -56,7 +55,7 @@ struct Lin1Prog {
     for (int j = 0; j < RowsOp::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsOp::row_of(j), t.rows - 1)];
     if (BWD) {
 #pragma unroll
-      for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
+      for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(t.mbase + 32 * i + acc_row(), t.rows - 1)];
     }
   }
   __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
@@ -83,7 +82,7 @@ struct Lin1Prog {
     const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      if (m_org[i] >= tc.rows) break;  // wave-uniform: no valid row in this fragment row
+      if (i >= tc.na) break;  // wave-uniform: no valid row in this fragment row
       float a[4][4], b[4][4];
 #pragma unroll
       for (int q = 0; q < 4; ++q)
@@ -92,10 +91,10 @@ struct Lin1Prog {
           a[q][e] = acc[0][i][4 * q + e];
           b[q][e] = acc[1][i][4 * q + e];
         }
-      // destination of 8 columns of tile row m_org[i]+row in a [*, ld] matrix, or nullptr
+      // destination of 8 columns of tile row (tc.mbase + 32 * i)+row in a [*, ld] matrix, or nullptr
       auto dst = [&](bf16* mat, int64_t ld, int col0, bool rows_lo_hi) {
         return [=, *this](int row, int col) -> bf16* {
-          const int rl = m_org[i] + row;
+          const int rl = (tc.mbase + 32 * i) + row;
           const int64_t r = (int64_t)tc.row0 + rl;
           if (rl >= tc.rows || j0 + col >= H) return nullptr;
           if (rows_lo_hi && (r < p.ab_lo || r >= p.ab_hi)) return nullptr;
@@ -131,7 +130,7 @@ struct Lin1Prog {
     float* red = (float*)epi;  // [4 column waves][BM]
     const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
     auto load_u = [&](int i, bf16x4 (&uq)[4]) {
-      const int64_t r = (int64_t)tc.row0 + min(m_org[i] + acc_row(), tc.rows - 1);
+      const int64_t r = (int64_t)tc.row0 + min((tc.mbase + 32 * i) + acc_row(), tc.rows - 1);
 #pragma unroll
       for (int q = 0; q < 4; ++q) uq[q] = *(const bf16x4*)(p.u + r * H + min(j0 + acc_col(q), H - 4));
     };
@@ -140,7 +139,7 @@ struct Lin1Prog {
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       gsums[i] = 0.0f;
-      if (m_org[i] >= tc.rows) continue;  // wave-uniform
+      if (i >= tc.na) continue;  // wave-uniform
       bf16x4 uq[4];
       load_u(i, uq);
       const float sv = g.sv[i];
@@ -166,7 +165,7 @@ struct Lin1Prog {
       }
       auto dst = [&](bf16* mat, int64_t ld, int col0) {
         return [=, *this](int row, int col) -> bf16* {
-          const int rl = m_org[i] + row;
+          const int rl = (tc.mbase + 32 * i) + row;
           const int64_t r = (int64_t)tc.row0 + rl;
           if (rl >= tc.rows || j0 + col >= H || r < p.ab_lo) return nullptr;
           return mat + r * ld + col0 + j0 + col;
@@ -179,7 +178,7 @@ struct Lin1Prog {
         stager.put(0, q, pack_bf16x4(acc[0][i][4 * q], acc[0][i][4 * q + 1], acc[0][i][4 * q + 2],
                                      acc[0][i][4 * q + 3]));
       stager.flush(dst(p.hs, H, 0));
-      gsums[i] = m_org[i] + acc_row() < tc.rows ? gsum : 0.0f;
+      gsums[i] = (tc.mbase + 32 * i) + acc_row() < tc.rows ? gsum : 0.0f;
     }
     // every wave is done with its staging area before the row sums overwrite it
     wait_lgkm0();
@@ -187,7 +186,8 @@ struct Lin1Prog {
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       const float gg = gsums[i] + __shfl_xor(gsums[i], 32);
-      if ((threadIdx.x & 63) < 32) red[wn * BM + m_org[i] + acc_row()] = gg;
+      // only the fragment rows this wave owns: the others belong to the other wave row
+      if (i < tc.na && (threadIdx.x & 63) < 32) red[wn * BM + (tc.mbase + 32 * i) + acc_row()] = gg;
     }
     wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
     __builtin_amdgcn_s_barrier();
@@ -208,11 +208,10 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   const int first_tile =
       p.h == nullptr && p.ab_lo > 0 ? TileSched::expert_tile_of_row(p.table, p.ab_lo) : 0;
   TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, first_tile);
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
-  Prog prog{p, p.D / kBK, wn, m_org, dyn_lds() + kStages * Ring::STAGE};
-  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
+  Prog prog{p, p.D / kBK, wn, dyn_lds() + kStages * Ring::STAGE};
+  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
 }
 
 struct Lin2Args {
@@ -233,12 +232,11 @@ struct Lin2Prog {
   };
   const Lin2Args& p;
   const int ktiles, wn;
-  const int (&m_org)[FM];
   RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) g.tok[i] = p.idx[t.row0 + min(m_org[i] + acc_row(), t.rows - 1)];
+    for (int i = 0; i < FM; ++i) g.tok[i] = p.idx[t.row0 + min(t.mbase + 32 * i + acc_row(), t.rows - 1)];
   }
   __device__ __forceinline__ void late(const TileCoord& t, Prep& g) const {
 #pragma unroll
@@ -256,7 +254,7 @@ struct Lin2Prog {
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      if (m_org[i] >= tc.rows) break;
+      if (i >= tc.na) break;
       const float sv = g.sv[i];
 #pragma unroll
       for (int f = 0; f < FN; ++f)
@@ -265,7 +263,7 @@ struct Lin2Prog {
           stager.put(f, q, pack_bf16x4(acc[f][i][4 * q] * sv, acc[f][i][4 * q + 1] * sv,
                                        acc[f][i][4 * q + 2] * sv, acc[f][i][4 * q + 3] * sv));
       stager.flush([&](int row, int col) -> bf16* {
-        const int rl = m_org[i] + row;
+        const int rl = (tc.mbase + 32 * i) + row;
         if (rl >= tc.rows || d0 + col >= D) return nullptr;
         return p.ys + ((int64_t)tc.row0 + rl) * D + d0 + col;
       });
@@ -276,11 +274,10 @@ struct Lin2Prog {
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
+  const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  Lin2Prog prog{p, p.H / kBK, wn, m_org, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, m_org, n_org);
+  Lin2Prog prog{p, p.H / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
 }
 
 // out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.

@@ -481,16 +481,16 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   ring.advance(ktiles);
 }
 
-// main loop for a wave that owns rows [m_org[0], m_org[0] + 32*FM) of a tile whose first
-// `rows` rows are valid.  `stores_pending`: the wave issued at least PENDING stores since the
-// first stages of this tile were requested (see wait_first_stage).
+// main loop for a wave that owns `na` fragment rows starting at tile row m_org[0].
+// `stores_pending`: the wave issued at least PENDING stores since the first stages of this
+// tile were requested (see wait_first_stage).
 template <class AOp, class BOp, int FM, int FN, int PENDING, class Hook>
 __device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                           StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                          const int (&n_org)[FN], int rows, bool stores_pending,
+                                          const int (&n_org)[FN], int na_, bool stores_pending,
                                           Hook hook) {
   static_assert(FM == 4, "dispatch written for 4 fragment rows per wave");
-  const int na = __builtin_amdgcn_readfirstlane(min(FM, max(0, (rows - m_org[0] + 31) >> 5)));
+  const int na = __builtin_amdgcn_readfirstlane(na_);
   if (na == 4) {
     if (PENDING > 0 && stores_pending)
       gemm_mainloop<AOp, BOp, FM, FN, 4, PENDING>(A, B, acc, ktiles, ring, m_org, n_org, hook);
@@ -565,7 +565,7 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
 // epilogue of tile t runs.
 template <int FM, int FN, class P, class AOp, class BOp>
 __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp>& ring,
-                                              const int (&m_org)[FM], const int (&n_org)[FN]) {
+                                              const int (&n_org)[FN]) {
   TileCoord c0 = sched.next();
   if (!c0.valid) return;
   TileCoord c1 = sched.next();
@@ -580,7 +580,8 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
     TileSched::Raw rn;
-    gemm_rows<AOp, BOp, FM, FN, 0>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.rows, false, [&] {
+    const int m_org[FM] = {c0.mbase, c0.mbase + 32, c0.mbase + 64, c0.mbase + 96};
+    gemm_rows<AOp, BOp, FM, FN, 0>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.na, false, [&] {
       prog.late(c0, p0);
       if (c1.valid) prog.gather(c1, p1);
       rn = sched.fetch();
