@@ -634,15 +634,19 @@ struct RowStager {
     return *(const bf16x8*)(st + row * PITCH + pc * 8);
   }
   // write everything put() since the last flush: dst(row, col) -> destination of 8 columns,
-  // or nullptr to drop them
-  template <class Dst>
+  // or nullptr to drop them.  STREAM: the data is not read again soon (weight gradients), so
+  // the stores are marked non-temporal and leave the kernel's inputs in the caches.
+  template <bool STREAM = false, class Dst>
   __device__ __forceinline__ void flush(Dst dst) const {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       int row, col;
       const bf16x8 v = get(p, row, col);
       bf16* d = dst(row, col);
-      if (d != nullptr) *(bf16x8*)d = v;
+      if (d != nullptr) {
+        if (STREAM) __builtin_nontemporal_store(v, (bf16x8*)d);
+        else *(bf16x8*)d = v;
+      }
     }
   }
 };

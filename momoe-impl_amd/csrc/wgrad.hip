@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
         for (int qd = 0; qd < 4; ++qd)
           stager.put(f, qd, pack_bf16x4(acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
                                         acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]));
-      stager.flush([&](int row, int col) -> bf16* {
+      stager.flush<true>([&](int row, int col) -> bf16* {
         const int x = tc.x0 + m_org[i] + row;
         if (x >= p.X || y0 + col >= p.Y) return nullptr;
         return out + (int64_t)x * p.Y + y0 + col;
