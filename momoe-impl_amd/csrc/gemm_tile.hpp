@@ -355,35 +355,25 @@ __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, 
   if (ktiles > 2) gemm_issue_head<2>(A, B, ring);
 }
 
-// Vector-memory operations of a wave complete in the order they were issued (loads and stores
-// share the one counter on this architecture), so "at most n outstanding" means "all but the
-// youngest n are done".  The waits below allow exactly the operations known to be younger than
-// the stage that is needed.  PENDING is a lower bound on the number of stores the wave issued
-// between requesting the first kFirst stages of this tile and entering its main loop (the
-// previous tile's epilogue): those sit between stage kFirst-1 and stage kFirst in the queue and
-// may stay in flight while the first stages are multiplied, instead of being drained first.
-template <int LOADS, int PENDING>
+// Waits on the transfers count operations: loads of a wave complete in the order they were
+// issued, so "at most n outstanding" means "all loads but the youngest n are done" (stores that
+// are still in flight only make the wait longer).  Each wait allows exactly the stages known
+// to have been requested after the one that is needed.
+template <int LOADS>
 __device__ __forceinline__ void wait_first_stage(int ktiles) {
-  static_assert((kFirst - 1) * LOADS + PENDING <= 63, "vmcnt is a 6-bit counter");
+  static_assert((kFirst - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
   static_assert(kFirst == 3 || kFirst == 4, "wait ladder written for 3 or 4 stages ahead");
-  if (kFirst == 4 && ktiles > 3) wait_vmcnt<3 * LOADS + PENDING>();
-  else if (ktiles > 2) wait_vmcnt<2 * LOADS + PENDING>();
-  else if (ktiles > 1) wait_vmcnt<LOADS + PENDING>();
-  else wait_vmcnt<PENDING>();
+  if (kFirst == 4 && ktiles > 3) wait_vmcnt<3 * LOADS>();
+  else if (ktiles > 2) wait_vmcnt<2 * LOADS>();
+  else if (ktiles > 1) wait_vmcnt<LOADS>();
+  else wait_vmcnt<0>();
 }
 // wait until the deposits of stage kt (>= 1) have landed, when the stages up to kt+kStages-2
 // have been requested and everything older than stage kt is known to be complete
-template <int LOADS, int PENDING>
+template <int LOADS>
 __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
-  static_assert((kStages - 2) * LOADS + PENDING <= 63, "vmcnt is a 6-bit counter");
+  static_assert((kStages - 2) * LOADS <= 63, "vmcnt is a 6-bit counter");
   static_assert(kStages == 4 || kStages == 5, "wait ladder written for 4 or 5 stages");
-  if (PENDING > 0 && kt < kFirst) {
-    if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS + PENDING>();
-    else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS + PENDING>();
-    else if (kt + 1 < ktiles) wait_vmcnt<LOADS + PENDING>();
-    else wait_vmcnt<PENDING>();
-    return;
-  }
   if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS>();
   else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
   else if (kt + 1 < ktiles) wait_vmcnt<LOADS>();
@@ -399,7 +389,7 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
 // under the whole main loop (they enter the vmcnt queue between two stages, which can only
 // make the stage waits err on the long side).  On return the ring has advanced to the next
 // tile; all buffers but the last stage's are free, other waves may still be reading that one.
-template <class AOp, class BOp, int FM, int FN, int NA, int PENDING, class Hook>
+template <class AOp, class BOp, int FM, int FN, int NA, class Hook>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                               StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
                                               const int (&n_org)[FN], Hook hook, int ktail = kBK) {
@@ -425,9 +415,9 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   // The scheduling fences keep the compiler from hoisting fragment reads across k-steps.
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
-  // Stage 0 has landed; every wave is done reading the previous tile, whose last buffer the
-  // next stage will reuse.
-  wait_first_stage<LOADS, PENDING>(ktiles);
+  // Stage 0 has landed (the previous tile's stores need not have); every wave is done reading
+  // the previous tile, whose last buffer the next stage will reuse.
+  wait_first_stage<LOADS>(ktiles);
   wait_lgkm0();
   __builtin_amdgcn_s_barrier();
   fence();
@@ -446,7 +436,7 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
     fence();
     // stage kt+1 has landed; all LDS reads of stage kt have returned, so its buffer may be
     // overwritten once every wave is past the barrier
-    wait_stage<LOADS, PENDING>(kt + 1, ktiles);
+    wait_stage<LOADS>(kt + 1, ktiles);
     wait_lgkm0();
     __builtin_amdgcn_s_barrier();
     fence();
@@ -481,26 +471,18 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   ring.advance(ktiles);
 }
 
-// main loop for a wave that owns `na` fragment rows starting at tile row m_org[0].
-// `stores_pending`: the wave issued at least PENDING stores since the first stages of this
-// tile were requested (see wait_first_stage).
-template <class AOp, class BOp, int FM, int FN, int PENDING, class Hook>
+// main loop for a wave that owns `na` fragment rows starting at tile row m_org[0]
+template <class AOp, class BOp, int FM, int FN, class Hook>
 __device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
                                           StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
-                                          const int (&n_org)[FN], int na_, bool stores_pending,
-                                          Hook hook) {
+                                          const int (&n_org)[FN], int na_, Hook hook) {
   static_assert(FM == 4, "dispatch written for 4 fragment rows per wave");
   const int na = __builtin_amdgcn_readfirstlane(na_);
-  if (na == 4) {
-    if (PENDING > 0 && stores_pending)
-      gemm_mainloop<AOp, BOp, FM, FN, 4, PENDING>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-    else
-      gemm_mainloop<AOp, BOp, FM, FN, 4, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  }
-  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else gemm_mainloop<AOp, BOp, FM, FN, 0, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  if (na == 4) gemm_mainloop<AOp, BOp, FM, FN, 4>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else gemm_mainloop<AOp, BOp, FM, FN, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
 }
 
 // the workgroup's dynamic LDS (size given at launch)
@@ -581,7 +563,7 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
     zero_acc<FM, FN>(acc);
     TileSched::Raw rn;
     const int m_org[FM] = {c0.mbase, c0.mbase + 32, c0.mbase + 64, c0.mbase + 96};
-    gemm_rows<AOp, BOp, FM, FN, 0>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.na, false, [&] {
+    gemm_rows<AOp, BOp, FM, FN>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.na, [&] {
       prog.late(c0, p0);
       if (c1.valid) prog.gather(c1, p1);
       rn = sched.fetch();

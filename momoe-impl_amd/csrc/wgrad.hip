@@ -32,8 +32,6 @@ struct WTile {
   bool valid;
 };
 
-constexpr int kTileStores = FM * RowStager<2>::PASSES;  // stores per lane in a full tile's epilogue
-
 constexpr int kEpilogueCost = 4;  // a tile's epilogue, in units of one k-stage of its main loop
 
 // Persistent workgroups.  id%8 is the XCD a workgroup lands on.  Tiles are numbered expert
@@ -127,19 +125,14 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
   WTile tc = next_tile();
   if (!tc.valid) return;
   start(tc);
-  bool stores_pending = false;  // a full tile's worth of stores was issued after start()
   while (true) {
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
     const int ktiles = (re - rb + kBK - 1) / kBK;  // rows of tc's expert (start(tc) ran last)
     const int ktail = re - rb - (ktiles - 1) * kBK;
     const WTile nx = next_tile();
-    if (ktiles > 0) {
-      if (stores_pending)
-        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, kTileStores>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
-      else
-        gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM, 0>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
-    }
+    if (ktiles > 0)
+      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
     if (nx.valid) start(nx);
 
     bf16* out = p.gw + (int64_t)tc.expert * p.X * p.Y;
@@ -158,8 +151,6 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
         return out + (int64_t)x * p.Y + y0 + col;
       });
     }
-    // every lane stored in every pass iff the tile lies fully inside the matrix
-    stores_pending = tc.x0 + BX <= p.X && tc.y0 + BY <= p.Y;
     if (!nx.valid) break;
     tc = nx;
   }
