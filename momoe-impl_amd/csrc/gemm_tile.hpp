@@ -254,11 +254,23 @@ struct TGatherDma {
   static_assert(kFirst == 3, "three cached stages");
 
   __device__ __forceinline__ Offs row_pairs(int kt) const {
+    static_assert(NCH == 2, "a wave's deposits of one stage cover four consecutive rows");
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r0 = row_begin + kt * kBK + w * (2 * NCH);
     Offs out;
+    if (gather != nullptr && r0 + 3 < row_end) {
+      // the four row ids sit next to each other: one scalar load instead of four
+      typedef int32_t i32x4 __attribute__((ext_vector_type(4), aligned(4)));
+      const i32x4 v = *(const i32x4 __attribute__((address_space(4)))*)(gather + r0);
+      out.a[0] = (uint32_t)v[0] * ldb;
+      out.b[0] = (uint32_t)v[1] * ldb;
+      out.a[1] = (uint32_t)v[2] * ldb;
+      out.b[1] = (uint32_t)v[3] * ldb;
+      return out;
+    }
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int ra = min(row_begin + kt * kBK + w * (2 * NCH) + j * 2, row_end - 1);
+      const int ra = min(r0 + j * 2, row_end - 1);
       const int rb = min(ra + 1, row_end - 1);
       out.a[j] = (uint32_t)(gather ? load_uniform(gather + ra) : ra - row_begin) * ldb;
       out.b[j] = (uint32_t)(gather ? load_uniform(gather + rb) : rb - row_begin) * ldb;
