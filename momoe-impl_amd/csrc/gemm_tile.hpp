@@ -18,16 +18,25 @@
 //           of those 4 k-rows.
 //
 // Sizing facts measured on MI355X that shape this file:
+//   * Under sustained MFMA load the chip is power-limited: a loop of nothing but this MFMA on
+//     random operands runs at 1.75 PFLOP/s with the shader clock at 1.73 GHz (2.3 PFLOP/s at
+//     2.4 GHz on zeros), the complete main loop at 1.6-1.7 GHz.  Time then follows the energy
+//     spent - multiplications, LDS and L2 traffic - far more than exposed latencies: useless
+//     work costs, idle cycles barely do.
 //   * LDS serves 16 lanes per clock: 256 B/clk for bank-conflict-free
-//     ds_read_b128, 128 B/clk for the transpose reads.
+//     ds_read_b128, 128 B/clk at best for the transpose reads.
 //   * A CU streams at most ~27 B/clk from L2 and ~19 B/clk from beyond it, and tile
-//     traffic of this shape sustains ~17 B/clk (10.5 TB/s over the chip), so the tile
-//     is 256x256, the largest the register file holds, and even then the loads, not
-//     the MFMA pipe, set the pace: several stages must be in flight at all times.
+//     traffic of this shape sustains ~19 B/clk (11.7 TB/s over the chip), which a 256x256 tile
+//     - the largest the register file holds - needs at ~60% of the MFMA peak: the loads
+//     set the pace as much as the MFMA pipe, and several stages must be in flight at all times.
+//   * The transfer instruction must take "uniform base + 32-bit lane offset": with a 64-bit
+//     address per lane a whole GEMM ran 20% slower.
 //   * Launching one 256x256 tile per workgroup costs ~25% in launch, pipeline fill
 //     and drain: workgroups are persistent and prefetch across tiles.
 //   * Rows of a ragged tile that do not exist are pointed at the last valid row: the 16
-//     lanes of a deposit then ask for one line instead of 16, which makes them nearly free.
+//     lanes of a deposit then ask for one line instead of 16.  What a small tile cannot avoid
+//     is streaming its whole weight block, so an expert's rows are cut into equal row tiles
+//     rather than full tiles plus a sliver.
 //
 // Global memory goes straight to LDS with global_load_lds_dwordx4 (no VGPR
 // staging): one wave instruction deposits 64 x 16 bytes contiguously.  Since
@@ -35,8 +44,8 @@
 // permuting WHICH 16-byte piece each lane fetches: rows keep their natural,
 // unpadded pitch, and the fragment reads above are bank-conflict free.  The same
 // freedom does all predication: a lane that would read outside the matrix is
-// pointed at a clamped row/column (results masked at the store) or, where exact
-// zeros are needed along k, at a 16-byte block of zeros.
+// pointed at a clamped row/column (results masked at the store; along k the main loop
+// zeroes the affected fragment registers instead).
 //
 // The k-loop runs a ring of 4 stages of 32 k: while one stage is multiplied (2 MFMA
 // k-steps) the next three are in flight; one s_barrier per stage.  The fragments of
@@ -62,10 +71,6 @@ constexpr int kKSteps = kBK / 16;  // MFMA k-steps per stage
 constexpr int kStages = 4;         // LDS ring depth
 constexpr int kFirst = 3;          // stages of a tile requested ahead of its main loop
 constexpr int kChunkElems = 512;   // one wave-wide 16-byte-per-lane deposit = 1 KiB
-
-static __device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0, 0, 0, 0};
-
-__device__ __forceinline__ const bf16* zero_chunk() { return (const bf16*)kZeroChunk; }
 
 // 16 bytes per lane, global -> LDS.  `lds_wave_base` is a wave-uniform LDS byte address; lane
 // L's bytes land at lds_wave_base + 16*L.  Completion is tracked by vmcnt.  Issued as inline
