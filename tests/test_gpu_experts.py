@@ -37,6 +37,9 @@ def test_tiny_reference_config(save_percent):
     (2048, 512, 384, 20, 6, 2, 1.8, 0),      # skew + shared experts, H = 1.5 column tiles
     (2048, 512, 384, 20, 6, 2, 1.8, 100),
     (16, 256, 128, 32, 4, 0, None, 0),       # decode-sized: most experts empty
+    (64, 64, 32, 1, 1, 0, None, 0),          # one expert, smallest supported D and H
+    (33, 96, 160, 5, 5, 0, None, 50),        # every token on every expert, odd token count
+    (700, 160, 96, 3, 2, 1, None, 0),        # experts taller than one tile, one shared expert
 ])
 def test_layer_parity(M, D, H, N, K, Ks, skew, sp):
     x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, Ks=Ks, seed=5, skew=skew)
