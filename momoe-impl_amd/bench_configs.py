@@ -1,0 +1,86 @@
+"""Timings of the other layer shapes of the benchmark plan on one MI355X: the Qwen3-shaped
+inference forward at several token counts, the skewed routing with shared experts, and the
+4096 x 2048 layer at save_percent 0 / 50 / 100.  (bench.py at the repository root measures
+the headline shape and prints the one JSON line the driver reads; this script prints a table.)
+
+Usage: python momoe-impl_amd/bench_configs.py
+"""
+import math
+import os
+import sys
+import time
+
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import momoe_amd  # noqa: E402
+from momoe_amd import _hip  # noqa: E402
+
+DEV = "cuda:0"
+
+
+def routing(M, N, K, Ks, skew, gen):
+    """mask_NM int32 [N,M], s_NM fp32 (transposed view): top-(K-Ks) of softmax(logits) over the
+    routed experts, renormalised; the last Ks experts hold every token."""
+    Ng = N - Ks
+    logits = torch.randn(M, N, generator=gen, device=DEV)
+    if skew:
+        logits[:, :Ng] -= skew * torch.log(torch.arange(1, Ng + 1, device=DEV, dtype=torch.float32))
+    p = torch.softmax(logits[:, :Ng], -1)
+    sel = torch.topk(p, K - Ks, dim=-1).indices
+    chosen = torch.zeros(M, Ng, dtype=torch.bool, device=DEV).scatter_(1, sel, True)
+    w = p * chosen
+    s_MN = torch.cat([w / w.sum(-1, keepdim=True), torch.softmax(logits[:, Ng:], -1)], -1)
+    mask = torch.ones(N, M, dtype=torch.int32, device=DEV)
+    mask[:Ng] = chosen.T.to(torch.int32)
+    return mask.contiguous(), s_MN.contiguous().T
+
+
+def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5):
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    x = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(1, M, D)
+    dy = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(1, M, D)
+    W1 = torch.empty(N, D, 2 * H, device=DEV, dtype=torch.bfloat16).normal_(0, 0.02, generator=gen)
+    W2 = torch.empty(N, H, D, device=DEV, dtype=torch.bfloat16).normal_(0, 0.02, generator=gen)
+    mask, s = routing(M, N, K, Ks, skew, gen)
+    layer = momoe_amd.MoMoE(D, H, N, K, sp, Wl1_ND2H=W1, Wl2_NHD=W2)
+
+    def fwd():
+        with torch.no_grad():
+            layer(x, mask, s)
+
+    def step():
+        xd, sd = x.detach().requires_grad_(), s.detach().requires_grad_()
+        y, _ = layer(xd, mask, sd)
+        y.backward(dy)
+        layer.Wl1_ND2H.grad = layer.Wl2_NHD.grad = None
+
+    def timeit(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    unit = float(D) * H * M * K
+    tf = timeit(fwd)
+    line = f"{name:30s} fwd {tf:8.3f} ms {6 * unit / tf / 1e9:6.0f} TF/s {M / tf * 1e3:11.0f} tok/s"
+    if backward:
+        torch.cuda.reset_peak_memory_stats()
+        tb = timeit(step)
+        line += (f" | fwd+bwd {tb:8.3f} ms {18 * unit / tb / 1e9:6.0f} TF/s {M / tb * 1e3:10.0f} tok/s"
+                 f" | peak {torch.cuda.max_memory_allocated() / 2**30:5.2f} GiB")
+    print(line, flush=True)
+
+
+if __name__ == "__main__":
+    assert torch.cuda.is_available() and _hip.abi_version() == 1
+    for M in (16, 128, 1024, 8192):
+        run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20)
+    run("headline D2048 H1024", 8192, 2048, 1024, 128, 8)
+    run("skewed + 4 shared, H1408", 16384, 2048, 1408, 64, 8, Ks=4, skew=1.5 * 1.2)
+    for sp in (0, 50, 100):
+        run(f"D4096 H2048, save_percent={sp}", 65536, 4096, 2048, 64, 8, sp=sp, steps=3)
