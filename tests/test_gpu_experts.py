@@ -48,6 +48,25 @@ def test_layer_parity(M, D, H, N, K, Ks, skew, sp):
     _check_all(dev, ref)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_small_shapes(seed):
+    # shapes drawn from a seeded generator: odd token counts, D and H any multiple of 32,
+    # few or many experts, shared experts, every save_percent regime
+    import random
+    rng = random.Random(1000 + seed)
+    D, H = 32 * rng.randint(1, 10), 32 * rng.randint(1, 10)
+    N = rng.randint(1, 40)
+    K = rng.randint(1, min(N, 6))
+    Ks = rng.randint(0, K - 1) if rng.random() < 0.4 else 0
+    M = rng.choice([1, 7, 64, 255, 256, 257, 600, 901])
+    sp = rng.choice([0, 0, 25, 50, 100])
+    skew = rng.choice([None, None, 1.5])
+    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, Ks=Ks, seed=seed, skew=skew)
+    dev = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
+    ref = run_oracle_layer(x, W1, W2, mask, s, dy)
+    _check_all(dev, ref)
+
+
 def test_experts_without_tokens_get_zero_weight_grads():
     M, D, H, N, K = 256, 128, 64, 8, 2
     x, W1, W2, _, _, dy = make_layer_inputs(M, D, H, N, K, seed=9)
