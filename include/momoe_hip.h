@@ -156,11 +156,22 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
  * Experts without rows get exact zeros.
  * Wl2 gradient: A = hs (X=H), B = G_y gathered by idx (Y=D).
  * Wl1 gradient: A = x gathered by idx (X=D), B = gz (Y=2H).
+ * workspace: device scratch (16-byte aligned, contents undefined on entry and exit) for
+ * fp32 partial tiles of MOMOE_WGRAD_PARTIAL_BYTES each.  An expert that holds many times
+ * the average number of rows is contracted in several pieces so that its tiles do not
+ * outlast everything else in the launch; the pieces meet in the workspace and a second
+ * kernel adds them.  Any size is accepted: momoe_wgrad_workspace_bytes() is the most the
+ * library will use, a smaller workspace means coarser pieces, 0 (workspace may be NULL)
+ * means none.  The result does not depend on the routing of other experts, but the
+ * summation order of a cut expert differs from that of an uncut one.
  */
+#define MOMOE_WGRAD_PARTIAL_BYTES 262144
+int64_t momoe_wgrad_workspace_bytes(int64_t N, int64_t X, int64_t Y, int64_t Msum);
 int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
                 const void* B_rows, int64_t ldb, const int32_t* b_gather,
                 const int32_t* cumsums_N1, void* GW_NXY,
-                int64_t M, int64_t N, int64_t X, int64_t Y, int64_t Msum, void* stream);
+                int64_t M, int64_t N, int64_t X, int64_t Y, int64_t Msum,
+                void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- router ----------------------------------------------------------------
  * momoe_router_fwd replaces the elementwise part of TopKRouterFunction.forward

@@ -3,7 +3,12 @@ inference forward at several token counts, the skewed routing with shared expert
 4096 x 2048 layer at save_percent 0 / 50 / 100.  (bench.py at the repository root measures
 the headline shape and prints the one JSON line the driver reads; this script prints a table.)
 
-Usage: python momoe-impl_amd/bench_configs.py
+Usage: python momoe-impl_amd/bench_configs.py            # the shapes above
+       python momoe-impl_amd/bench_configs.py --chart    # the grid of the reference's README charts
+                                                         # (momoe/images/moe_full.png, moe_forward.png,
+                                                         # moe_memory.png): TF/s forward and
+                                                         # forward+backward at save_percent 0/50/100 and
+                                                         # the memory held between forward and backward
 """
 import math
 import os
@@ -34,6 +39,15 @@ def routing(M, N, K, Ks, skew, gen):
     mask = torch.ones(N, M, dtype=torch.int32, device=DEV)
     mask[:Ng] = chosen.T.to(torch.int32)
     return mask.contiguous(), s_MN.contiguous().T
+
+
+def balanced_routing(M, N, K, gen):
+    """Every expert gets exactly M*K/N tokens: token m goes to experts m + j*N/K (mod N)."""
+    assert N % K == 0
+    cols = (torch.arange(M, device=DEV)[:, None] + torch.arange(K, device=DEV)[None, :] * (N // K)) % N
+    chosen = torch.zeros(M, N, dtype=torch.bool, device=DEV).scatter_(1, cols, True)
+    w = torch.rand(M, N, generator=gen, device=DEV) * chosen
+    return chosen.T.to(torch.int32).contiguous(), (w / w.sum(-1, keepdim=True)).contiguous().T
 
 
 def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5):
@@ -76,8 +90,72 @@ def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5):
     print(line, flush=True)
 
 
+def chart_row(B, S, D, H, N, K, kind, steps=5):
+    """One configuration of the reference's charts: forward TF/s, forward+backward TF/s at
+    save_percent 0 / 50 / 100 and, per save_percent, the bytes alive after forward that were
+    not alive before it plus x itself (what the reference's memory chart plots: x, y and the
+    tensors saved for backward; weights, mask and gates excluded)."""
+    M = B * S
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    x = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(B, S, D)
+    dy = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(B, S, D)
+    W1 = torch.empty(N, D, 2 * H, device=DEV, dtype=torch.bfloat16).normal_(0, 0.02, generator=gen)
+    W2 = torch.empty(N, H, D, device=DEV, dtype=torch.bfloat16).normal_(0, 0.02, generator=gen)
+    if kind == "balanced":
+        mask, s = balanced_routing(M, N, K, gen)
+    else:
+        mask, s = routing(M, N, K, 0, 1.8 if kind == "skewed" else None, gen)
+    unit = float(D) * H * M * K
+    cells = []
+    for sp in (0, 50, 100):
+        layer = momoe_amd.MoMoE(D, H, N, K, sp, Wl1_ND2H=W1, Wl2_NHD=W2)
+
+        def fwd():
+            with torch.no_grad():
+                layer(x, mask, s)
+
+        def step(measure=False):
+            xd, sd = x.detach().requires_grad_(), s.detach().requires_grad_()
+            before = torch.cuda.memory_allocated()
+            y, _ = layer(xd, mask, sd)
+            held = torch.cuda.memory_allocated() - before + x.numel() * 2
+            y.backward(dy)
+            del y
+            layer.Wl1_ND2H.grad = layer.Wl2_NHD.grad = None
+            return held
+
+        def timeit(fn):
+            for _ in range(2):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps * 1e3
+
+        tf, tb = timeit(fwd), timeit(step)
+        held = step()
+        cells.append(f"sp{sp:3d}: fwd {6 * unit / tf / 1e9:5.0f} f+b {18 * unit / tb / 1e9:5.0f} TF/s"
+                     f" held {held / 1e9:5.2f} GB")
+        del layer
+    print(f"{B},{S},{D},{H},{N},{K} {kind:8s} | " + " | ".join(cells), flush=True)
+
+
+CHART_GRID = [
+    (2, 512, 1024, 512, 32, 4, "balanced"), (4, 2048, 2048, 1024, 64, 8, "balanced"),
+    (4, 2048, 2048, 1024, 64, 8, "skewed"), (6, 2048, 2048, 1280, 64, 6, "random"),
+    (4, 1920, 2176, 1152, 64, 6, "random"), (8, 4096, 2048, 1024, 128, 8, "balanced"),
+    (8, 4096, 2048, 1024, 128, 8, "skewed"), (8, 8192, 2048, 1024, 128, 8, "balanced"),
+]
+
+
 if __name__ == "__main__":
     assert torch.cuda.is_available() and _hip.abi_version() == 1
+    if "--chart" in sys.argv[1:]:
+        for row in CHART_GRID:
+            chart_row(*row)
+        sys.exit(0)
     for M in (16, 128, 1024, 8192):
         run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20)
     run("headline D2048 H1024", 8192, 2048, 1024, 128, 8)

@@ -38,13 +38,14 @@ struct TileCoord {
 
 // Persistent-workgroup iterator over the (row tile, column block) pairs of a grouped GEMM.
 // Workgroups are dealt round-robin to the 8 XCDs, so id%8 selects the XCD; each XCD owns one
-// contiguous eighth of the (expert-major, column-block, row-tile-minor) sequence and its
+// contiguous eighth of the tile sequence (expert-major; the order inside an expert is given at resolve()) and its
 // workgroups walk it with a stride of gridDim/8.  All tiles of an expert therefore run on
 // one XCD close together in time and share its L2 for both the expert's weights and its
 // token rows.
 // A tile is looked up in two steps so that the table read can travel while other work runs:
 // fetch() issues the scalar loads of the workgroup's next tile, resolve() does the arithmetic.
 struct TileSched {
+  static constexpr int kBandTiles = 4;
   struct Raw {
     int q, expert, first, rstart, mi;
     bool any;
@@ -90,9 +91,16 @@ struct TileSched {
     // long and stay in step, and no tile streams a whole weight block for a handful of rows.
     const int nt = (r.mi + bm - 1) / bm;
     const int th = ((r.mi + nt - 1) / nt + 31) & ~31;
+    // Order inside an expert: bands of kBandTiles row tiles, each band crossing every column
+    // block before the next band starts (row tile fastest inside a band).  The workgroups of
+    // an XCD hold consecutive positions at any moment, so they share a few row tiles and a few
+    // weight blocks in L2 however many rows the expert has.
     const int qq = r.q - r.first * nb;
-    const int tl = qq % nt;
-    tc.tn = qq / nt;
+    const int band = qq / (kBandTiles * nb);
+    const int in_band = qq - band * (kBandTiles * nb);
+    const int band_rows = min(kBandTiles, nt - band * kBandTiles);
+    const int tl = band * kBandTiles + in_band % band_rows;
+    tc.tn = in_band / band_rows;
     tc.expert = r.expert;
     tc.row0 = r.rstart + tl * th;
     tc.rows = min(th, r.mi - tl * th);

@@ -46,7 +46,9 @@ _SIGNATURES = {
                                       _i64, _i64, _i64, _i64, _p]),
     "momoe_gs_scatter": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _p]),
     "momoe_dgrad_x": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
-    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "momoe_wgrad_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p,
+                           _i64, _p]),
     "momoe_router_fwd": (_int, [_p, _int, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p]),
     "momoe_router_bwd": (_int, [_p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p]),
 }
@@ -211,11 +213,20 @@ def dgrad_x(gz, Wl1_ND2H, table, gxs, M):
                               gz.shape[0], _stream())
 
 
-def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, M, Msum):
+def wgrad_workspace_bytes(N, X, Y, Msum):
+    return _lib.momoe_wgrad_workspace_bytes(N, X, Y, Msum)
+
+
+def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, M, Msum, workspace_bytes=None):
+    """workspace_bytes: scratch for the partial tiles of experts with many rows; default = the
+    most the library can use for this shape, 0 = never cut an expert."""
     N, X, Y = GW_NXY.shape
+    if workspace_bytes is None:
+        workspace_bytes = wgrad_workspace_bytes(N, X, Y, Msum)
+    ws = torch.empty(workspace_bytes, device=GW_NXY.device, dtype=torch.uint8) if workspace_bytes else None
     _call("momoe_wgrad", _ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
                             B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X,
-                            Y, Msum, _stream())
+                            Y, Msum, _ptr(ws), workspace_bytes, _stream())
 
 
 # ---------------------------------------------------------------- router

@@ -121,16 +121,21 @@ class MoEFunction(torch.autograd.Function):
                 _hip.gs_scatter(gs_part, idx, cumsums, G_s)
             del gs_part
 
+            # scratch for the weight gradients of experts with many rows: what the library can
+            # use, but no more than u occupied (just freed, so the peak does not move)
+            ws_cap = hs.numel() * hs.element_size()
             G_W2 = None
             if need_w2:
                 G_W2 = torch.empty_like(W2)
-                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, M, msum)
+                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, M, msum,
+                           workspace_bytes=min(ws_cap, _hip.wgrad_workspace_bytes(N, H, D, msum)))
             del hs
 
             G_W1 = None
             if need_w1:
                 G_W1 = torch.empty_like(W1)
-                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, M, msum)
+                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, M, msum,
+                           workspace_bytes=min(ws_cap, _hip.wgrad_workspace_bytes(N, D, 2 * H, msum)))
 
             G_x_BSD = None
             if need_x:

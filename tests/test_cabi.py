@@ -49,7 +49,13 @@ def test_size_queries_and_argument_validation(lib):
     # null pointers / bad sizes are rejected on the host before anything is launched
     z = ctypes.c_void_p(0)
     assert lib.momoe_combine(z, z, z, i64(1), i64(8), i64(1), i64(1), z) == 1
-    assert lib.momoe_wgrad(z, i64(8), z, z, i64(8), z, z, z, i64(1), i64(1), i64(8), i64(8), i64(1), z) == 1
+    assert lib.momoe_wgrad(z, i64(8), z, z, i64(8), z, z, z, i64(1), i64(1), i64(8), i64(8), i64(1),
+                           z, i64(0), z) == 1
+    lib.momoe_wgrad_workspace_bytes.restype = ctypes.c_int64
+    # at most 8 partial tiles of 256 KiB per workgroup (256), fewer when there are few rows
+    assert lib.momoe_wgrad_workspace_bytes(i64(128), i64(2048), i64(2048), i64(65536)) == 2048 * 262144
+    assert lib.momoe_wgrad_workspace_bytes(i64(2), i64(64), i64(64), i64(9000)) == 4 * 262144
+    assert lib.momoe_wgrad_workspace_bytes(i64(2), i64(64), i64(64), i64(100)) == 0
 
 
 def test_host_modules_refuse_cpu_tensors():

@@ -40,6 +40,9 @@ def test_tiny_reference_config(save_percent):
     (64, 64, 32, 1, 1, 0, None, 0),          # one expert, smallest supported D and H
     (33, 96, 160, 5, 5, 0, None, 50),        # every token on every expert, odd token count
     (700, 160, 96, 3, 2, 1, None, 0),        # experts taller than one tile, one shared expert
+    (9000, 64, 96, 3, 2, 1, None, 0),        # a shared expert with enough rows that its weight
+                                             # gradient is contracted in several pieces
+    (12000, 96, 64, 6, 1, 0, 1.8, 50),       # one routed expert holds most rows
 ])
 def test_layer_parity(M, D, H, N, K, Ks, skew, sp):
     x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, Ks=Ks, seed=5, skew=skew)
@@ -65,6 +68,41 @@ def test_random_small_shapes(seed):
     dev = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
     ref = run_oracle_layer(x, W1, W2, mask, s, dy)
     _check_all(dev, ref)
+
+
+@pytest.mark.parametrize("gather_a", [True, False])
+def test_weight_gradient_of_cut_experts(gather_a):
+    # experts of 20000 / 3 / 0 / 5000 rows: the first is contracted in pieces that meet in the
+    # fp32 workspace.  Checked against a plain fp32 matmul per expert and against the same
+    # launch without a workspace (no expert is cut then).
+    from momoe_amd import _hip
+    dev = "cuda:0"
+    sizes = [20000, 3, 0, 5000]
+    N, X, Y, M = len(sizes), 320, 512, 20000
+    msum = sum(sizes)
+    g = torch.Generator(device=dev).manual_seed(11)
+    cumsums = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32, device=dev)
+    A = torch.randn(M if gather_a else msum, X, generator=g, device=dev).to(torch.bfloat16)
+    B = torch.randn(msum if gather_a else M, Y, generator=g, device=dev).to(torch.bfloat16)
+    ids = torch.cat([torch.randperm(M, generator=g, device=dev)[:n].sort().values for n in sizes]).to(torch.int32)
+    ga, gb = (ids, None) if gather_a else (None, ids)
+    need = _hip._lib.momoe_wgrad_workspace_bytes(N, X, Y, msum)
+    assert need >= 3 * 4 * 262144
+    out = {}
+    for ws in (need, 262144 * 16, 0):
+        GW = torch.full((N, X, Y), float("nan"), device=dev, dtype=torch.bfloat16)
+        _hip.wgrad(A, ga, B, gb, cumsums, GW, M, msum, workspace_bytes=ws)
+        out[ws] = GW.float()
+    torch.cuda.synchronize()
+    for e, n in enumerate(sizes):
+        r0 = int(cumsums[e])
+        Ae = A[ids[r0:r0 + n].long()] if gather_a else A[r0:r0 + n]
+        Be = B[r0:r0 + n] if gather_a else B[ids[r0:r0 + n].long()]
+        want = Ae.float().T @ Be.float()
+        for ws, got in out.items():
+            assert_close(got[e].cpu(), want.cpu(), f"GW[{e}] ws={ws}", rel=5e-3)
+    assert torch.equal(out[0][2], torch.zeros(X, Y, device=dev))
+    assert torch.equal(out[need][1:3], out[0][1:3])  # uncut experts: bit-identical
 
 
 def test_experts_without_tokens_get_zero_weight_grads():
