@@ -23,10 +23,10 @@ PEAK_HBM_GBS = 8000.0
 # (profiles/momoe_layer_headline_{fetch,write}_size.txt; fetch scaled x2.0, write x1.0 by the
 # 256 MiB copy in the same runs); None for a kernel that has not been measured.
 MEASURED_TRAFFIC_BYTES = {
-    "momoe_lin1_swiglu_fwd": 2 * 819631 * 1024 + 173810 * 1024,
-    "momoe_lin1_swiglu_bwd": 2 * 920033 * 1024 + 397929 * 1024,
-    "momoe_wgrad[Wl1]": 2 * 297466 * 1024 + 1048599 * 1024,
-    "momoe_dgrad_x": 2 * 800659 * 1024 + 262144 * 1024,
+    "momoe_lin1_swiglu_fwd": 2 * 814482 * 1024 + 173802 * 1024,
+    "momoe_lin1_swiglu_bwd": 2 * 924177 * 1024 + 398073 * 1024,
+    "momoe_wgrad[Wl1]": 2 * 298640 * 1024 + 1048603 * 1024,
+    "momoe_dgrad_x": 2 * 801241 * 1024 + 262144 * 1024,
 }
 
 
