@@ -123,3 +123,33 @@ def test_training_smoke_loss_decreases():
         losses.append(loss.item())
     assert 0.5 < losses[0] < 1.5
     assert losses[-1] < 0.9 * losses[0]
+
+
+def test_training_smoke_at_the_reference_size():
+    # momoe/test.py as written: B,S,D,H = 4,8192,1024,512; N,K,Ks = 32,6,1; 10 warm-up forwards,
+    # then 200 AdamW steps (lr 1e-3) on mean((y - x)^2).  Its docstring is the only expected
+    # result the reference states: the loss starts around 1 and goes down towards 0.
+    import momoe_amd
+    torch.manual_seed(0)
+    B, S, D, H, N, K, Ks = 4, 8192, 1024, 512, 32, 6, 1
+    x = torch.randn(B, S, D, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    moe = momoe_amd.MoE(D, H, N, K, Ks, save_percent=0, bias_update_rate=1e-4)
+    for _ in range(10):
+        moe(x)
+    opt = torch.optim.AdamW(moe.parameters(), lr=1e-3)
+    losses = []
+    for _ in range(200):
+        x.grad = torch.zeros_like(x)
+        y = moe(x)
+        loss = torch.mean(torch.square(y.float() - x.float()))
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        losses.append(loss.item())
+    assert all(l == l for l in losses), "loss became NaN"
+    assert 0.8 < losses[0] < 1.2
+    assert losses[-1] < 0.5 * losses[0]
+    assert losses[-1] == min(losses[-20:]) or losses[-1] < 1.05 * min(losses[-20:])
+    # the routed experts' selection bias moved by at most 210 steps of the update rate
+    b = moe.biases_N[:N - Ks]
+    assert torch.all(b.abs() <= 210 * 1e-4 + 1e-6) and torch.all(torch.isinf(moe.biases_N[N - Ks:]))
