@@ -43,6 +43,12 @@ def _compare(mask, K, out):
     (16, 128, 8, 0, None),      # decode-sized
     (1, 4, 4, 0, None),
     (65536, 64, 8, 0, None),    # largest token count of the configurations
+    # one token panel (M <= 256)
+    (256, 128, 8, 0, None),     # a full panel
+    (200, 300, 7, 2, None),     # 19 expert groups, two shared experts
+    (255, 1024, 6, 0, 1.8),     # many experts, few tokens
+    (256, 1025, 3, 0, None),    # N one past a multiple of the 16-expert panel
+    (77, 17, 17, 0, None),      # every token on every expert, N just over one group
 ])
 def test_index_bit_exact(M, N, K, Ks, skew):
     mask, _ = make_routing(M, N, K, Ks, seed=11, skew=skew)
@@ -64,6 +70,27 @@ def test_violation_counter_and_no_out_of_bounds():
     bad[0:6, 9] = 1        # token 9 has more than K
     out = _run(bad, 4)
     assert out["violations"].item() >= 2
+
+
+def test_violations_single_panel():
+    mask, _ = make_routing(100, 40, 4, seed=4)
+    bad = mask.clone()
+    bad[:, 5] = 0          # token 5 has no expert
+    bad[0:6, 9] = 1        # token 9 has more than K
+    out = _run(bad, 4)
+    assert out["violations"].item() >= 2
+    # too many pairs in total: the tile table is emptied so that the GEMMs do nothing
+    over = torch.ones(40, 100, dtype=torch.int32)
+    out = _run(over, 4)
+    assert out["violations"].item() >= 1 and out["tile_table"][0].item() == 0
+
+
+def test_strided_mask_single_panel():
+    mask, _ = make_routing(130, 24, 3, seed=2)
+    strided = mask.T.contiguous().to("cuda:0").T  # strides (1, N)
+    from momoe_amd import _hip
+    out = {k: v.cpu() for k, v in _hip.index_build(strided, 3).items()}
+    _compare(mask, 3, out)
 
 
 def test_experts_without_tokens():
