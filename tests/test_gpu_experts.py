@@ -221,3 +221,57 @@ def test_skewed_routing_with_shared_experts_full_size():
 def test_memory_stress_layer_full_size(sp):
     # D=4096, H=2048, N=64, K=8, 65536 tokens: 524288 sorted rows, 4 GiB intermediates
     _sampled_parity_on_device_inputs(65536, 4096, 2048, 64, 8, 0, None, sp, 16, experts=(63,), n_tok=8)
+
+
+def test_input_formats_and_partial_gradients():
+    # what a caller may hand over besides the router's own outputs: fp32 x (cast to bf16 like
+    # the reference, momoe/momoe.py:863), non-contiguous x and G_y, a contiguous s_NM, a strided
+    # mask; and backward with only some inputs requiring gradients.
+    import momoe_amd
+    M, D, H, N, K = 384, 128, 96, 10, 3
+    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, seed=21)
+    ref = run_oracle_layer(x, W1, W2, mask, s, dy)
+    dev = "cuda:0"
+    layer = momoe_amd.MoMoE(D, H, N, K, 0, Wl1_ND2H=W1.to(dev), Wl2_NHD=W2.to(dev))
+    # the oracle sees bf16-rounded x: hand the device the same values as fp32, in a strided view
+    x32 = x.to(torch.bfloat16).float()
+    wide = torch.zeros(M, 2 * D, device=dev)
+    wide[:, ::2] = x32.to(dev)
+    xd = wide[:, ::2].reshape(2, M // 2, D).requires_grad_()
+    assert not xd.is_contiguous() or xd.dtype == torch.float32
+    sd = s.contiguous().to(dev).requires_grad_()                      # plain [N, M]
+    maskd = mask.T.contiguous().to(dev).T                             # strides (1, N)
+    y, sizes = layer(xd, maskd, sd)
+    assert y.dtype == torch.bfloat16 and y.shape == (2, M // 2, D) and sizes.dtype == torch.int64
+    dy_wide = torch.zeros(2, M // 2, 2 * D, device=dev, dtype=torch.bfloat16)
+    dy_wide[..., ::2] = dy.to(dev, torch.bfloat16).reshape(2, M // 2, D)
+    y.backward(dy_wide[..., ::2])
+    torch.cuda.synchronize()
+    assert torch.equal(sizes.cpu(), ref["sizes"])
+    assert_close(y.reshape(M, D), ref["y"], "y")
+    assert_close(xd.grad.reshape(M, D), ref["G_x"], "G_x")
+    assert_close(sd.grad, ref["G_s"], "G_s")
+    assert_close(layer.Wl1_ND2H.grad, ref["G_W1"], "G_W1")
+    assert_close(layer.Wl2_NHD.grad, ref["G_W2"], "G_W2")
+
+    # frozen experts: only x and s get gradients; then only the weights
+    frozen = momoe_amd.MoMoE(D, H, N, K, 50, Wl1_ND2H=W1.to(dev), Wl2_NHD=W2.to(dev))
+    for p in frozen.parameters():
+        p.requires_grad_(False)
+    xb = x.to(dev, torch.bfloat16).reshape(1, M, D).requires_grad_()
+    sb = s.contiguous().to(dev).requires_grad_()
+    yb, _ = frozen(xb, mask.to(dev), sb)
+    yb.backward(dy.to(dev, torch.bfloat16).reshape(1, M, D))
+    assert frozen.Wl1_ND2H.grad is None and frozen.Wl2_NHD.grad is None
+    assert_close(xb.grad.reshape(M, D), ref["G_x"], "G_x (frozen experts)")
+    assert_close(sb.grad, ref["G_s"], "G_s (frozen experts)")
+    xc = x.to(dev, torch.bfloat16).reshape(1, M, D)
+    yc, _ = layer(xc, mask.to(dev), s.contiguous().to(dev))
+    layer.zero_grad(set_to_none=True)
+    yc.backward(dy.to(dev, torch.bfloat16).reshape(1, M, D))
+    assert_close(layer.Wl1_ND2H.grad, ref["G_W1"], "G_W1 (weights only)")
+    assert_close(layer.Wl2_NHD.grad, ref["G_W2"], "G_W2 (weights only)")
+    # no_grad forward keeps nothing for a backward
+    with torch.no_grad():
+        yn, _ = layer(xc, mask.to(dev), s.contiguous().to(dev))
+    assert not yn.requires_grad and torch.equal(yn, yc.detach())
