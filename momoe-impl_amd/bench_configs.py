@@ -4,6 +4,7 @@ inference forward at several token counts, the skewed routing with shared expert
 the headline shape and prints the one JSON line the driver reads; this script prints a table.)
 
 Usage: python momoe-impl_amd/bench_configs.py            # the shapes above
+       python momoe-impl_amd/bench_configs.py --only skewed   # one of: inference headline skewed large
        python momoe-impl_amd/bench_configs.py --chart    # the grid of the reference's README charts
                                                          # (momoe/images/moe_full.png, moe_forward.png,
                                                          # moe_memory.png): TF/s forward and
@@ -156,9 +157,14 @@ if __name__ == "__main__":
         for row in CHART_GRID:
             chart_row(*row)
         sys.exit(0)
-    for M in (16, 128, 1024, 8192):
-        run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20)
-    run("headline D2048 H1024", 8192, 2048, 1024, 128, 8)
-    run("skewed + 4 shared, H1408", 16384, 2048, 1408, 64, 8, Ks=4, skew=1.5 * 1.2)
-    for sp in (0, 50, 100):
-        run(f"D4096 H2048, save_percent={sp}", 65536, 4096, 2048, 64, 8, sp=sp, steps=3)
+    only = sys.argv[sys.argv.index("--only") + 1] if "--only" in sys.argv[1:] else None
+    if only in (None, "inference"):
+        for M in (16, 128, 1024, 8192):
+            run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20)
+    if only in (None, "headline"):
+        run("headline D2048 H1024", 8192, 2048, 1024, 128, 8)
+    if only in (None, "skewed"):
+        run("skewed + 4 shared, H1408", 16384, 2048, 1408, 64, 8, Ks=4, skew=1.5 * 1.2)
+    if only in (None, "large"):
+        for sp in (0, 50, 100):
+            run(f"D4096 H2048, save_percent={sp}", 65536, 4096, 2048, 64, 8, sp=sp, steps=3)
