@@ -1,5 +1,4 @@
-"""Build libmomoe_hip.so (gfx950) from csrc/*.hip with hipcc, in-tree, and the stand-alone
-measurement tools of probes/*.hip (one executable each, next to its source).
+"""Build libmomoe_hip.so (gfx950) from csrc/*.hip with hipcc, in-tree.
 
 Usage: python build.py
 """
@@ -53,24 +52,6 @@ def build_library(verbose=True):
     return LIB
 
 
-def build_probes(verbose=True):
-    """One executable per probes/*.hip (measurement tools; the library does not use them)."""
-    pdir = os.path.join(HERE, "probes")
-    built = []
-    for f in sorted(os.listdir(pdir)):
-        if not f.endswith(".hip"):
-            continue
-        exe = os.path.join(pdir, f[:-4])
-        r = subprocess.run([_hipcc(), *FLAGS, "-o", exe, os.path.join(pdir, f)], capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed for {f}:\n{r.stderr}")
-        built.append(exe)
-    if verbose:
-        print(f"built {len(built)} probe(s): {', '.join(os.path.basename(b) for b in built)}")
-    return built
-
-
 if __name__ == "__main__":
     build_library()
-    build_probes()
     sys.exit(0)
