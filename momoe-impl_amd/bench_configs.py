@@ -107,7 +107,7 @@ def chart_row(B, S, D, H, N, K, kind, steps=5):
     else:
         mask, s = routing(M, N, K, 0, 1.8 if kind == "skewed" else None, gen)
     unit = float(D) * H * M * K
-    cells = []
+    cells, result = [], {}
     for sp in (0, 50, 100):
         layer = momoe_amd.MoMoE(D, H, N, K, sp, Wl1_ND2H=W1, Wl2_NHD=W2)
 
@@ -137,10 +137,13 @@ def chart_row(B, S, D, H, N, K, kind, steps=5):
 
         tf, tb = timeit(fwd), timeit(step)
         held = step()
+        result[sp] = {"fwd_tflops": 6 * unit / tf / 1e9, "fwd_bwd_tflops": 18 * unit / tb / 1e9,
+                      "held_bytes": held}
         cells.append(f"sp{sp:3d}: fwd {6 * unit / tf / 1e9:5.0f} f+b {18 * unit / tb / 1e9:5.0f} TF/s"
                      f" held {held / 1e9:5.2f} GB")
         del layer
     print(f"{B},{S},{D},{H},{N},{K} {kind:8s} | " + " | ".join(cells), flush=True)
+    return result
 
 
 CHART_GRID = [

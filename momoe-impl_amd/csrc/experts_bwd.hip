@@ -89,20 +89,33 @@ struct SavedArgs {
   float* gs_part;
   int nparts;
   int64_t msum;
-  int H, N;
+  int H, N, M;
 };
 
 __global__ __launch_bounds__(256) void swiglu_bwd_saved_kernel(SavedArgs p) {
   const int64_t r = blockIdx.x;
   const int H = p.H;
   __shared__ float s_red[4];
+  if (r >= p.cumsums[p.N]) {
+    // The routing holds fewer pairs than M*K (a token with fewer than K experts): this sorted
+    // row does not exist and its token id was never written.  Its outputs are defined zeros.
+    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
+      *(bf16x8*)(p.gz + r * 2 * H + c) = z;
+      *(bf16x8*)(p.gz + r * 2 * H + H + c) = z;
+      *(bf16x8*)(p.hs + r * H + c) = z;
+    }
+    for (int q = threadIdx.x; q < p.nparts; q += 256) p.gs_part[(int64_t)q * p.msum + r] = 0.0f;
+    return;
+  }
   // expert of row r: the i with cumsums[i] <= r < cumsums[i+1]
   int lo = 0, hi = p.N;
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
     if (p.cumsums[mid] <= r) lo = mid; else hi = mid;
   }
-  const float sv = p.s[(int64_t)lo * p.ssn + (int64_t)p.idx[r] * p.ssm];
+  const int tok = min(max(p.idx[r], 0), p.M - 1);
+  const float sv = p.s[(int64_t)lo * p.ssn + (int64_t)tok * p.ssm];
   const bf16* a_row = p.ab + r * 2 * H;
   const bf16* u_row = p.u + r * H;
   float gsum = 0.0f;
@@ -251,11 +264,12 @@ extern "C" int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH, 
     return MOMOE_ERR_BAD_ARG;
   if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_Msum2H) || !aligned16(hs_MsumH))
     return MOMOE_ERR_BAD_ARG;
-  if (H % 8 != 0 || Msum >= (1ll << 31) || nparts > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
+  if (H % 8 != 0 || Msum >= (1ll << 31) || M >= (1ll << 31) || nparts > (1 << 20))
+    return MOMOE_ERR_UNSUPPORTED;
   if (Msave == 0) return MOMOE_OK;
   SavedArgs a{(const bf16*)ab_save, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m, idx_Msum,
               cumsums_N1, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part, (int)nparts, Msum, (int)H,
-              (int)N};
+              (int)N, (int)M};
   swiglu_bwd_saved_kernel<<<(unsigned)Msave, 256, 0, (hipStream_t)stream>>>(a);
   return launch_status();
 }

@@ -66,7 +66,8 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
 __global__ __launch_bounds__(1024) void index_scan_kernel(
     int32_t* __restrict__ part, int N, int NC, int64_t msum_cap,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums,
-    int32_t* __restrict__ table, int tile_rows, int32_t* __restrict__ violations) {
+    int32_t* __restrict__ table, int tile_rows, int32_t* __restrict__ violations,
+    int32_t* __restrict__ idx, int32_t* __restrict__ which) {
   __shared__ int32_t s_size[kMaxExperts];
   __shared__ int32_t s_cum[kMaxExperts];
   __shared__ int32_t s_first[kMaxExperts];
@@ -107,6 +108,7 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
       const bool overflow = (int64_t)run_rows > msum_cap;
       if (overflow) atomicAdd(violations, 1);
       s_total[0] = overflow ? 0 : run_tiles;
+      s_total[1] = run_rows;
       table[0] = overflow ? 0 : run_tiles;
       table[1] = tile_rows;
       table[2] = 0;
@@ -114,6 +116,12 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
     }
   }
   __syncthreads();
+  // A routing with fewer than M*K pairs leaves the sorted rows past the last pair without a
+  // token: give them token 0 / slot 0, so that nothing downstream reads an undefined id.
+  for (int64_t r = (int64_t)s_total[1] + t; r < msum_cap; r += 1024) {
+    idx[r] = 0;
+    which[r] = 0;
+  }
   if (s_total[0] == 0) return;
   for (int i = t; i < N; i += 1024) {
     const int v = s_size[i];
@@ -168,7 +176,11 @@ __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
       ++k;
     }
   }
-  if (m < M && g == gridDim.y - 1 && k != K) atomicAdd(violations, 1);
+  if (m < M && g == gridDim.y - 1 && k != K) {
+    atomicAdd(violations, 1);
+    // slots the token does not fill: -1 = "no row" (momoe_combine skips them)
+    for (int kk = k; kk < K; ++kk) inv[(int64_t)m * K + kk] = -1;
+  }
 }
 
 }  // namespace
@@ -208,7 +220,7 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
   index_count_kernel<<<grid, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N,
                                                     NC, part, tokcnt);
   index_scan_kernel<<<1, 1024, 0, st>>>(part, (int)N, NC, M * K, sizes_N, cumsums_N1, tile_table,
-                                        tile_rows, violations);
+                                        tile_rows, violations, idx_Msum, which_Msum);
   index_scatter_kernel<<<grid, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N,
                                                       (int)K, NC, part, tokcnt, cumsums_N1,
                                                       idx_Msum, which_Msum, inv_MK, violations);

@@ -16,6 +16,15 @@ import torch.nn as nn
 from . import _hip
 
 
+# The layer requires every token to be routed to exactly K experts (momoe/momoe.py:831, the
+# reference's README) and, like the reference, does not verify it: the index build counts the
+# offending tokens on the device and reading that counter would stall the host.  With too few
+# pairs the missing contributions are simply absent from y and the gradients; with too many the
+# tile list is emptied and y is undefined.  Set CHECK_ROUTING = True to read the counter after
+# every forward (one device synchronisation per call) and raise on a violation.
+CHECK_ROUTING = False
+
+
 def _saved_rows(msum, save_percent):
     # momoe/momoe.py:251
     return int(msum * save_percent / 100.0)
@@ -60,7 +69,8 @@ class MoEFunction(torch.autograd.Function):
             ib = _hip.index_build(mask, K)
             idx, table = ib["idx_Msum"], ib["tile_table"]
             msum = M * K
-            msave = _saved_rows(msum, save_percent)
+            # nothing is kept for a backward that cannot happen (no input wants a gradient)
+            msave = _saved_rows(msum, save_percent) if any(ctx.needs_input_grad[:5]) else 0
 
             h = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
             ab_save = torch.empty((msave, 2 * H), device=dev, dtype=torch.bfloat16) if msave > 0 else None
@@ -79,7 +89,9 @@ class MoEFunction(torch.autograd.Function):
         if ab_save is not None:
             saved.append(ab_save)
         ctx.save_for_backward(*saved)
-        ctx.routing_violations = ib["violations"]
+        if CHECK_ROUTING and int(ib["violations"].item()) != 0:
+            raise RuntimeError(f"mask_NM: {int(ib['violations'].item())} tokens do not have exactly K = {K} "
+                               "experts (or the mask holds more than M*K pairs)")
         sizes_N = ib["sizes_N"]
         ctx.mark_non_differentiable(sizes_N)
         return y_MD.view(B, S, D).to(device=x_BSD.device), sizes_N
@@ -182,5 +194,6 @@ class MoMoE(nn.Module):
     def forward(self, x_BSD, mask_NM, s_NM):
         """x_BSD [B,S,D]; mask_NM int32 0/1 [N,M] with exactly K ones per token; s_NM [N,M]
         gate weights (zero off-mask).  Returns (y_BSD bf16, tokens per expert int64 [N])."""
-        return MoEFunction.apply(x_BSD, self.Wl1_ND2H, self.Wl2_NHD, mask_NM, s_NM, self.K,
-                                 self.save_percent)
+        # pre-activations are only worth keeping when a backward can follow
+        sp = self.save_percent if torch.is_grad_enabled() else 0
+        return MoEFunction.apply(x_BSD, self.Wl1_ND2H, self.Wl2_NHD, mask_NM, s_NM, self.K, sp)

@@ -148,7 +148,7 @@ def experts_forward_dense(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, dtype=torch.fl
 # experts: backward in closed form (the formulas the device kernels implement)
 # --------------------------------------------------------------------------
 def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
-                                 dtype=torch.float64):
+                                 dtype=torch.float64, reference_rounding=False):
     """Gradients of `experts_forward` written out by hand.
 
     Restates `swiglu_backward_kernel` (momoe/momoe.py:470-535),
@@ -162,7 +162,16 @@ def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
       G_W1_i = x[tok]^T @ [G_a | G_b]         (:730-737)
       G_x[tok] += [G_a | G_b] @ W1_i^T        (:667-681, :754)
       G_s[i,tok] = sum_d G_y[tok,d] * ypre[d] (:699-703), zero elsewhere (:721)
+
+    `reference_rounding` rounds through bf16 the three intermediates that the
+    reference itself stores as bf16 before they enter a weight-gradient GEMM:
+    Gy' (:340, the `G_y_MsumD` buffer of :551), the recomputed h (:533-535) and
+    G_z (:527-531, `G_z_Msum2H` of :555).  Everything else stays in `dtype`.
+    It exists to measure how far the reference's OWN arithmetic is from the
+    unrounded result (tests/test_oracle_experts.py); parity tests compare
+    against the unrounded form.
     """
+    rnd = (lambda t: t.to(torch.bfloat16).to(dtype)) if reference_rounding else (lambda t: t)
     x = x_MD.to(dtype)
     W1 = Wl1_ND2H.to(dtype)
     W2 = Wl2_NHD.to(dtype)
@@ -186,12 +195,12 @@ def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
         h = a * b * sig
         ypre = h @ W2[i]
         gy = Gy[tok]
-        gys = gy * s[i, tok][:, None]
+        gys = rnd(gy * s[i, tok][:, None])
         G_h = gys @ W2[i].T
         G_a = G_h * b * sig
         G_b = G_h * a * sig * (1 + b * (1 - sig))
-        G_z = torch.cat([G_a, G_b], dim=1)
-        G_W2[i] = h.T @ gys
+        G_z = rnd(torch.cat([G_a, G_b], dim=1))
+        G_W2[i] = rnd(h).T @ gys
         G_W1[i] = xi.T @ G_z
         G_x.index_add_(0, tok, G_z @ W1[i].T)
         G_s[i, tok] = (gy * ypre).sum(dim=1)
@@ -201,7 +210,7 @@ def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
 # --------------------------------------------------------------------------
 # router
 # --------------------------------------------------------------------------
-def router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, logits=None):
+def router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, logits=None, forced_mask_NM=None):
     """Top-k + softmax router with a selection bias and shared experts.
 
     Restates `TopKRouterFunction.forward` (momoe/topk_router.py:85-124):
@@ -215,7 +224,10 @@ def router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, logits=None):
     the [M,N] weight matrix (:120).
 
     `logits` (fp32 [M,N]) may be supplied to bypass the matmul, e.g. to feed
-    tie-free fp32 logits.
+    tie-free fp32 logits.  `forced_mask_NM` replaces the top-k selection by a
+    given one (its routed rows): bf16 logits contain exact ties whose order
+    torch.topk leaves unspecified, so a test that wants the same routing on
+    both sides hands over the selection it checked to be a valid top-k.
     Returns dict with mask_NM, s_NM, p_sel_MN (the masked softmax
     probabilities the backward needs, :106), Ng_M, Ks_M, logits_MN.
     """
@@ -226,9 +238,12 @@ def router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, logits=None):
     p_g = torch.softmax(logits[:, :Ng], dim=-1, dtype=torch.float32)
     p_s = torch.softmax(logits[:, Ng:], dim=-1, dtype=torch.float32)
     sel_scores = p_g + biases_N.to(torch.float32)[:Ng][None, :]
-    _, sel = torch.topk(sel_scores, K - Ks, dim=-1)
-    sel_mask = torch.zeros((M, Ng), dtype=torch.bool)
-    sel_mask.scatter_(1, sel, True)
+    if forced_mask_NM is None:
+        _, sel = torch.topk(sel_scores, K - Ks, dim=-1)
+        sel_mask = torch.zeros((M, Ng), dtype=torch.bool)
+        sel_mask.scatter_(1, sel, True)
+    else:
+        sel_mask = forced_mask_NM[:Ng].T != 0
     p_sel = p_g * sel_mask
     Ng_M = p_sel.sum(dim=-1)
     Ks_M = p_s.sum(dim=-1)
@@ -242,6 +257,7 @@ def router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, logits=None):
         "Ng_M": Ng_M,
         "Ks_M": Ks_M,
         "logits_MN": logits,
+        "sel_scores_MNg": sel_scores,
     }
 
 
@@ -339,10 +355,10 @@ class _OracleRouterFn(torch.autograd.Function):
     """Router with the reference's backward (fixed selection, closed form)."""
 
     @staticmethod
-    def forward(ctx, x_BSD, Wg_DN, biases_N, N, K, Ks):
+    def forward(ctx, x_BSD, Wg_DN, biases_N, N, K, Ks, forced_mask_NM=None):
         B, S, D = x_BSD.shape
         x_MD = x_BSD.reshape(B * S, D)
-        r = router_forward(x_MD, Wg_DN, biases_N, N, K, Ks)
+        r = router_forward(x_MD, Wg_DN, biases_N, N, K, Ks, forced_mask_NM=forced_mask_NM)
         ctx.save_for_backward(x_MD, Wg_DN, r["mask_NM"], r["p_sel_MN"], r["s_NM"], r["Ng_M"], r["Ks_M"])
         ctx.Ks = Ks
         ctx.mark_non_differentiable(r["mask_NM"])
@@ -356,7 +372,8 @@ class _OracleRouterFn(torch.autograd.Function):
         Wg = Wg_DN.to(torch.float32)
         G_x = G_x_BSD.reshape(x_MD.shape).to(torch.float32) + G_logit @ Wg.T
         G_Wg = x_MD.to(torch.float32).T @ G_logit
-        return G_x.reshape(G_x_BSD.shape).to(G_x_BSD.dtype), G_Wg.to(Wg_DN.dtype), None, None, None, None
+        return (G_x.reshape(G_x_BSD.shape).to(G_x_BSD.dtype), G_Wg.to(Wg_DN.dtype), None, None, None,
+                None, None)
 
 
 class OracleTopKRouter(nn.Module):
@@ -368,9 +385,11 @@ class OracleTopKRouter(nn.Module):
         if Wg_DN is None:
             Wg_DN = torch.randn(self.D, self.N) / self.D
         self.Wg_DN = nn.Parameter(Wg_DN.clone().detach().to(torch.bfloat16))
+        self.forced_mask_NM = None  # tests: use this selection instead of torch.topk's
 
     def forward(self, x_BSD, biases_N):
-        return _OracleRouterFn.apply(x_BSD, self.Wg_DN, biases_N, self.N, self.K, self.Ks)
+        return _OracleRouterFn.apply(x_BSD, self.Wg_DN, biases_N, self.N, self.K, self.Ks,
+                                     self.forced_mask_NM)
 
 
 class OracleMoE(nn.Module):

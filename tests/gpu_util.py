@@ -12,25 +12,42 @@ def rel_err(got, ref):
     return ((got - ref).norm() / ref.norm().clamp_min(1e-30)).item()
 
 
-def assert_close(got, ref, what, rel=1e-2):
-    """Elementwise |got-ref| <= ATOL*max(1, rms(ref)) + RTOL*|ref| and a norm-wise bound.
-
-    For tensors whose RMS is at most 1 (y, G_x, G_s and the weight gradients of small
-    experts) this is the plain rtol/atol 2e-2 check.  The absolute term follows the RMS
-    of larger tensors (per expert for the weight gradients) because the bf16 rounding of the MFMA inputs of the weight-gradient
-    GEMMs (G_z and h are bf16 in the reference too, momoe/momoe.py:555-556) accumulates
-    over the contraction and scales with the result itself.
-    """
+def tolerance_report(got, ref):
+    """(elements outside the plain rtol/atol 2e-2 check, elements outside the check whose
+    absolute term is scaled by max(1, rms(ref)), the scale used, relative L2 error)."""
     got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
-    e = rel_err(got, ref)
     if ref.dim() == 3:  # per-expert weight gradients: each expert has its own scale
         scale = ref.pow(2).mean(dim=(1, 2), keepdim=True).sqrt().clamp_min(1.0)
     else:
         scale = max(1.0, ref.pow(2).mean().sqrt().item())
-    bad = (got - ref).abs() > ATOL * scale + RTOL * ref.abs()
-    assert not bad.any(), (f"{what}: {int(bad.sum())}/{bad.numel()} elements outside tolerance, "
-                           f"max abs diff {(got - ref).abs().max().item():.4g}, rms(ref) "
-                           f"{ref.pow(2).mean().sqrt().item():.4g}, relative L2 error {e:.3e}")
+    diff = (got - ref).abs()
+    plain = int((diff > ATOL + RTOL * ref.abs()).sum())
+    scaled = int((diff > ATOL * scale + RTOL * ref.abs()).sum())
+    return plain, scaled, scale, rel_err(got, ref)
+
+
+def assert_close(got, ref, what, rel=1e-2):
+    """Elementwise |got-ref| <= ATOL*max(1, rms(ref)) + RTOL*|ref| and a norm-wise bound.
+
+    For tensors whose RMS is at most 1 (y, G_x, and the weight gradients of small experts)
+    this is the plain rtol/atol 2e-2 check.  The absolute term follows the RMS of larger
+    tensors (per expert for the weight gradients): the operands of the weight-gradient GEMMs
+    (G_z, h, the scaled G_y) are bf16 in the reference too (momoe/momoe.py:340, 533-535, 555),
+    their rounding accumulates over the contraction and scales with the result itself, so the
+    reference's own arithmetic misses the plain check on those tensors by the same margin
+    (tests/test_oracle_experts.py::test_reference_rounding_alone_breaks_the_plain_tolerance).
+    Whenever the scaling matters, the number of elements outside the PLAIN check is printed
+    (pytest -rP / -s shows it).
+    """
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    plain, scaled, _, e = tolerance_report(got, ref)
+    if plain:
+        print(f"[tolerance] {what}: {plain}/{ref.numel()} elements outside plain rtol/atol 2e-2, "
+              f"{scaled} outside the RMS-scaled check; rms(ref) {ref.pow(2).mean().sqrt().item():.3g}, "
+              f"relative L2 error {e:.2e}")
+    assert scaled == 0, (f"{what}: {scaled}/{ref.numel()} elements outside tolerance, "
+                         f"max abs diff {(got - ref).abs().max().item():.4g}, rms(ref) "
+                         f"{ref.pow(2).mean().sqrt().item():.4g}, relative L2 error {e:.3e}")
     assert e < rel, f"{what}: relative L2 error {e:.3e} >= {rel}"
 
 
@@ -65,3 +82,64 @@ def run_oracle_layer(x, W1, W2, mask, s, dy, dtype=torch.float32):
     y.backward(r(dy))
     return {"y": y.detach(), "G_x": xo.grad, "G_W1": W1o.grad, "G_W2": W2o.grad, "G_s": so.grad,
             "sizes": (mask != 0).sum(1).to(torch.int64)}
+
+
+def device_layer_inputs(M, D, H, N, K, Ks=0, skew=None, seed=77, routing_seed=3):
+    """x, dy, Wl1, Wl2 drawn on the GPU in bf16 (the host would take minutes at the full
+    sizes) plus CPU routing (mask_NM, s_NM) from `helpers.make_routing`."""
+    from helpers import make_routing
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(seed)
+    x = torch.randn(M, D, generator=g, device=dev).to(torch.bfloat16)
+    dy = torch.randn(M, D, generator=g, device=dev).to(torch.bfloat16)
+    W1 = torch.empty(N, D, 2 * H, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
+    W2 = torch.empty(N, H, D, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
+    mask, s = make_routing(M, N, K, Ks, seed=routing_seed, skew=skew)
+    return x, dy, W1, W2, mask, s
+
+
+def oracle_forward_for_tokens(x, W1, W2, mask, s, tok):
+    """Oracle forward for the tokens `tok` (CPU index tensor) of device-resident x / weights,
+    restricted to the experts those tokens use.  Returns (y fp32 [len(tok), D], the fp32 copy
+    of x[tok] with requires_grad set, so the caller can continue into the backward)."""
+    f = lambda t: t.detach().float().cpu()
+    dev = x.device
+    used = torch.nonzero(mask[:, tok].sum(1)).flatten()
+    xs = f(x[tok.to(dev)]).requires_grad_()
+    yo = oracle.experts_forward(xs, f(W1[used.to(dev)]), f(W2[used.to(dev)]), mask[used][:, tok],
+                                s[used][:, tok])
+    return yo, xs
+
+
+def sampled_parity_on_device_inputs(M, D, H, N, K, Ks, skew, sp, B, experts, n_tok=16):
+    """Full-size layer forward + backward; the oracle sees the same bits, copied back for a
+    sample of tokens and experts only."""
+    import momoe_amd
+    dev = "cuda:0"
+    x, dy, W1, W2, mask, s = device_layer_inputs(M, D, H, N, K, Ks, skew)
+    layer = momoe_amd.MoMoE(D, H, N, K, sp, Wl1_ND2H=W1, Wl2_NHD=W2)
+    xd = x.reshape(B, M // B, D).clone().requires_grad_()
+    sd = s.T.contiguous().to(dev).T.requires_grad_()
+    y, sizes = layer(xd, mask.to(dev), sd)
+    y.backward(dy.reshape(B, M // B, D))
+    torch.cuda.synchronize()
+    assert torch.equal(sizes.cpu(), (mask != 0).sum(1))
+    assert torch.isfinite(y).all() and torch.isfinite(xd.grad).all()
+    assert torch.isfinite(layer.Wl1_ND2H.grad).all() and torch.isfinite(layer.Wl2_NHD.grad).all()
+    f = lambda t: t.detach().float().cpu()
+    # sampled tokens: forward and dL/dx against the oracle restricted to the experts they use
+    tok = torch.arange(0, M, M // n_tok)[:n_tok]
+    yo, xs = oracle_forward_for_tokens(x, W1, W2, mask, s, tok)
+    assert_close(y.reshape(M, D)[tok.to(dev)], yo, "y (sampled tokens)")
+    yo.backward(f(dy[tok.to(dev)]))
+    assert_close(xd.grad.reshape(M, D)[tok.to(dev)], xs.grad, "G_x (sampled tokens)")
+    # sampled experts: weight gradients and dL/ds from the closed form
+    for i in experts:
+        sel = torch.nonzero(mask[i]).flatten()
+        one = torch.ones(1, sel.numel(), dtype=torch.int32)
+        _, gW1, gW2, gs = oracle.experts_backward_closed_form(
+            f(x[sel.to(dev)]), f(W1[i:i + 1]), f(W2[i:i + 1]), one, s[i:i + 1, sel], f(dy[sel.to(dev)]),
+            dtype=torch.float32)
+        assert_close(layer.Wl1_ND2H.grad[i], gW1[0], f"G_W1[{i}]")
+        assert_close(layer.Wl2_NHD.grad[i], gW2[0], f"G_W2[{i}]")
+        assert_close(sd.grad[i, sel.to(dev)], gs[0], f"G_s[{i}]")

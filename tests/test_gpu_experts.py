@@ -5,7 +5,8 @@ import pytest
 import torch
 
 import oracle
-from gpu_util import assert_close, rel_err, run_device_layer, run_oracle_layer
+from gpu_util import (assert_close, rel_err, run_device_layer, run_oracle_layer,
+                      sampled_parity_on_device_inputs as _sampled_parity_on_device_inputs)
 from helpers import make_layer_inputs
 
 pytestmark = pytest.mark.gpu
@@ -168,56 +169,19 @@ def test_headline_shape_properties_and_sampled_parity():
     assert_close(xd.grad.reshape(M, D)[tok], xs.grad, "G_x (sampled tokens)")
 
 
-def _sampled_parity_on_device_inputs(M, D, H, N, K, Ks, skew, sp, B, experts, n_tok=16):
-    """Full-size layer whose x / weights / dy are drawn on the GPU (the host would take minutes
-    at these sizes); the oracle sees the same bits, copied back for a sample of tokens and
-    experts only."""
-    import momoe_amd
-    from helpers import make_routing
-    dev = "cuda:0"
-    g = torch.Generator(device=dev).manual_seed(77)
-    x = torch.randn(M, D, generator=g, device=dev).to(torch.bfloat16)
-    dy = torch.randn(M, D, generator=g, device=dev).to(torch.bfloat16)
-    W1 = torch.empty(N, D, 2 * H, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
-    W2 = torch.empty(N, H, D, device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=g)
-    mask, s = make_routing(M, N, K, Ks, seed=3, skew=skew)
-    layer = momoe_amd.MoMoE(D, H, N, K, sp, Wl1_ND2H=W1, Wl2_NHD=W2)
-    xd = x.reshape(B, M // B, D).clone().requires_grad_()
-    sd = s.T.contiguous().to(dev).T.requires_grad_()
-    y, sizes = layer(xd, mask.to(dev), sd)
-    y.backward(dy.reshape(B, M // B, D))
-    torch.cuda.synchronize()
-    assert torch.equal(sizes.cpu(), (mask != 0).sum(1))
-    assert torch.isfinite(y).all() and torch.isfinite(xd.grad).all()
-    assert torch.isfinite(layer.Wl1_ND2H.grad).all() and torch.isfinite(layer.Wl2_NHD.grad).all()
-    f = lambda t: t.detach().float().cpu()
-    # sampled tokens: forward and dL/dx against the oracle restricted to the experts they use
-    tok = torch.arange(0, M, M // n_tok)[:n_tok]
-    used = torch.nonzero(mask[:, tok].sum(1)).flatten()
-    xs = f(x[tok.to(dev)]).requires_grad_()
-    yo = oracle.experts_forward(xs, f(W1[used.to(dev)]), f(W2[used.to(dev)]), mask[used][:, tok], s[used][:, tok])
-    assert_close(y.reshape(M, D)[tok.to(dev)], yo, "y (sampled tokens)")
-    yo.backward(f(dy[tok.to(dev)]))
-    assert_close(xd.grad.reshape(M, D)[tok.to(dev)], xs.grad, "G_x (sampled tokens)")
-    # sampled experts: weight gradients and dL/ds from the closed form
-    for i in experts:
-        sel = torch.nonzero(mask[i]).flatten()
-        one = torch.ones(1, sel.numel(), dtype=torch.int32)
-        _, gW1, gW2, gs = oracle.experts_backward_closed_form(
-            f(x[sel.to(dev)]), f(W1[i:i + 1]), f(W2[i:i + 1]), one, s[i:i + 1, sel], f(dy[sel.to(dev)]),
-            dtype=torch.float32)
-        assert_close(layer.Wl1_ND2H.grad[i], gW1[0], f"G_W1[{i}]")
-        assert_close(layer.Wl2_NHD.grad[i], gW2[0], f"G_W2[{i}]")
-        assert_close(sd.grad[i, sel.to(dev)], gs[0], f"G_s[{i}]")
-
-
 def test_skewed_routing_with_shared_experts_full_size():
     # D=2048, H=1408, 60 routed + 4 shared experts, 4 routed + 4 shared per token, 16384 tokens,
     # Zipf-like load: a few experts hold ~10x the mean, the shared ones hold every token
     _sampled_parity_on_device_inputs(16384, 2048, 1408, 64, 8, 4, 1.8, 0, 8, experts=(0, 59))
 
 
-@pytest.mark.parametrize("sp", [0, 50])
+def test_headline_layer_full_size_with_everything_saved():
+    # the headline layer at save_percent=100: every row takes the saved-pre-activation branch
+    # of the SwiGLU backward (momoe/momoe.py:486-491)
+    _sampled_parity_on_device_inputs(8192, 2048, 1024, 128, 8, 0, None, 100, 4, experts=(0, 77, 127))
+
+
+@pytest.mark.parametrize("sp", [0, 50, 100])
 def test_memory_stress_layer_full_size(sp):
     # D=4096, H=2048, N=64, K=8, 65536 tokens: 524288 sorted rows, 4 GiB intermediates
     _sampled_parity_on_device_inputs(65536, 4096, 2048, 64, 8, 0, None, sp, 16, experts=(63,), n_tok=8)

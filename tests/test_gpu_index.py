@@ -100,3 +100,24 @@ def test_experts_without_tokens():
     out = _run(mask, 2)
     _compare(mask, 2, out)
     assert out["sizes_N"].tolist() == [0, 300, 0, 0, 0, 0, 300, 0]
+
+
+def test_routing_with_missing_pairs_leaves_nothing_undefined():
+    # tokens with fewer than K experts: the sorted rows past the last pair get token 0 / slot 0
+    # and the token's unused slots of inv_MK say "no row" (-1)
+    M, N, K = 600, 20, 4
+    mask, _ = make_routing(M, N, K, seed=8)
+    short = mask.clone()
+    short[:, 17] = 0
+    for m in (3, 300, 599):
+        short[int(torch.nonzero(short[:, m])[-1]), m] = 0
+    out = _run(short, K)
+    o = oracle.index_build(short)
+    total = int(o["cumsums_N"][-1])
+    assert total == M * K - K - 3 and out["violations"].item() == 4
+    for k in ("sizes_N", "cumsums_N"):
+        assert np.array_equal(out[k].numpy(), o[k]), k
+    assert np.array_equal(out["idx_Msum"].numpy()[:total], o["idx_Msum"])
+    assert np.array_equal(out["which_Msum"].numpy()[:total], o["which_Msum"])
+    assert np.all(out["idx_Msum"].numpy()[total:] == 0) and np.all(out["which_Msum"].numpy()[total:] == 0)
+    assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])  # the oracle writes -1 for missing pairs

@@ -90,3 +90,35 @@ def test_module_signature_and_outputs():
     m = oracle.OracleMoMoE(D, H, N, K, save_percent=0, Wl1_ND2H=W1, Wl2_NHD=W2)
     y, sizes = m(x.reshape(2, 16, D), mask, s)
     assert y.shape == (2, 16, D) and sizes.dtype == torch.int64 and sizes.sum() == M * K
+
+
+@pytest.mark.parametrize("rows", [512, 4096])
+def test_reference_rounding_alone_breaks_the_plain_tolerance(rows):
+    # One expert with `rows` tokens: the weight gradients contract over `rows`.  The reference
+    # stores the operands of those GEMMs as bf16 (scaled G_y, recomputed h, G_z:
+    # momoe/momoe.py:340, 533-535, 555).  fp32 arithmetic with just those three roundings,
+    # against the unrounded fp64 result, already leaves elements of the weight gradients
+    # outside rtol/atol 2e-2 once their RMS exceeds 1 -- while every element stays inside the
+    # check whose absolute term is scaled by the RMS (the one the GPU parity tests use) and
+    # the other gradients stay inside the plain check.
+    from gpu_util import tolerance_report
+    g = torch.Generator().manual_seed(rows)
+    D, H = 128, 64
+    r = lambda t: t.to(torch.bfloat16).float()
+    x = r(torch.randn(rows, D, generator=g))
+    W1 = r(torch.randn(1, D, 2 * H, generator=g) * 0.09)  # a, b ~ N(0, 1) like the headline layer
+    W2 = r(torch.randn(1, H, D, generator=g) * 0.09)
+    dy = r(torch.randn(rows, D, generator=g))
+    mask = torch.ones(1, rows, dtype=torch.int32)
+    s = torch.rand(1, rows, generator=g) * 0.5 + 0.1
+    exact = oracle.experts_backward_closed_form(x, W1, W2, mask, s, dy, dtype=torch.float64)
+    rounded = oracle.experts_backward_closed_form(x, W1, W2, mask, s, dy, dtype=torch.float32,
+                                                  reference_rounding=True)
+    report = {n: tolerance_report(gt, ex) for n, gt, ex in zip(("G_x", "G_W1", "G_W2", "G_s"), rounded, exact)}
+    for n in ("G_W1", "G_W2"):
+        plain, scaled, scale, rel = report[n]
+        assert float(scale.max()) > 2.0       # the tensors the scaling is meant for
+        assert plain > 0, (n, report[n])      # the reference's own rounding misses the plain check
+        assert scaled == 0 and rel < 5e-3     # and passes the scaled one with room
+    for n in ("G_x", "G_s"):
+        assert report[n][0] == 0 and report[n][1] == 0
