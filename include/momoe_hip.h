@@ -9,8 +9,10 @@
  *   - work is only ENQUEUED on `stream` (a hipStream_t passed as void*); no entry
  *     point synchronises with the device.
  *   - the return value is a status code (MOMOE_OK or MOMOE_ERR_*); no C++
- *     exception crosses the boundary.  Entry points are re-entrant and keep no
- *     global mutable state.
+ *     exception crosses the boundary.  Entry points are re-entrant; the only state the
+ *     library keeps is set once and never changed afterwards (the raised dynamic-LDS
+ *     limit of each GEMM kernel, the per-device address of the fixed scratch array of
+ *     momoe_index_build_static).
  *   - dimension letters: M tokens, D embedding, H expert hidden, N experts,
  *     K experts per token, Msum = M*K (token,expert) pairs = "sorted rows":
  *     the rows of expert i occupy [cumsums[i], cumsums[i+1]) in ascending token order.
@@ -65,6 +67,27 @@ int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m
                       int32_t* tile_table, int tile_rows,
                       void* workspace, int64_t workspace_bytes,
                       int32_t* violations, void* stream);
+
+/* momoe_index_build_static: momoe_index_build without the workspace arguments, for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The panel counts
+ * go to a fixed array of MOMOE_INDEX_STATIC_SCRATCH_BYTES that is part of the library's device
+ * code (each GPU the library runs on holds it until the process ends), so the call allocates
+ * nothing and calls no allocating routine; inputs and outputs are still the caller's.
+ * momoe_index_workspace_bytes(M, N) > MOMOE_INDEX_STATIC_SCRATCH_BYTES (e.g. M = 65536 tokens
+ * with more than 240 experts) returns MOMOE_ERR_UNSUPPORTED.  Results are bit-identical to
+ * momoe_index_build.  All calls on one GPU share that GPU's array: two calls that overlap on one
+ * GPU (different streams) race; calls on one stream, or on different GPUs, do not.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress), which must not happen
+ * under stream capture: make one call per device beforehand.
+ */
+#define MOMOE_INDEX_STATIC_SCRATCH_BYTES 4194304
+int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m,
+                             int64_t M, int64_t N, int64_t K,
+                             int64_t* sizes_N, int32_t* cumsums_N1, int32_t* idx_Msum,
+                             int32_t* which_Msum, int32_t* inv_MK,
+                             int32_t* tile_table, int tile_rows,
+                             int32_t* violations, void* stream);
 
 /* ---- experts forward -----------------------------------------------------
  * momoe_lin1_swiglu_fwd replaces lin1_kernel (momoe/momoe.py:69-152):

@@ -11,6 +11,8 @@
 //   pass 3 (scatter): per panel, each set bit learns its sorted row
 //                     (expert base + panel base + wave base + rank in ballot) and
 //                     its slot (set bits of the token in earlier experts).
+#include <mutex>
+
 #include "common.hpp"
 
 namespace momoe {
@@ -225,4 +227,52 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
                                                       (int)K, NC, part, tokcnt, cumsums_N1,
                                                       idx_Msum, which_Msum, inv_MK, violations);
   return launch_status();
+}
+
+// ---- the same without a caller-provided workspace ------------------------------------------
+// The panel counts live in a fixed array in device memory that is part of the library's code
+// object: every GPU the library runs on holds its own copy, at its own address, until the
+// process ends.  In host code the array's NAME is only a handle for the runtime, not a device
+// address: the address is looked up once per device and kept; kernels and every other use of
+// the array's memory take that pointer.
+namespace {
+constexpr int64_t kStaticScratchBytes = MOMOE_INDEX_STATIC_SCRATCH_BYTES;
+__attribute__((used)) static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device d, once looked up
+
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MOMOE_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return MOMOE_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MOMOE_OK;
+}
+}  // namespace
+
+extern "C" int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m,
+                                        int64_t M, int64_t N, int64_t K, int64_t* sizes_N,
+                                        int32_t* cumsums_N1, int32_t* idx_Msum,
+                                        int32_t* which_Msum, int32_t* inv_MK, int32_t* tile_table,
+                                        int tile_rows, int32_t* violations, void* stream) {
+  if (M <= 0 || N <= 0) return MOMOE_ERR_BAD_ARG;
+  // sizes beyond the fixed array are refused, never truncated
+  if (momoe_index_workspace_bytes(M, N) > kStaticScratchBytes) return MOMOE_ERR_UNSUPPORTED;
+  void* ws = nullptr;
+  const int st = scratch_of_current_device(&ws);
+  if (st != MOMOE_OK) return st;
+  // Every word of the array that the scatter pass reads was written by the count pass of the
+  // same call, so nothing has to be cleared between calls.
+  return momoe_index_build(mask_NM, stride_n, stride_m, M, N, K, sizes_N, cumsums_N1, idx_Msum,
+                           which_Msum, inv_MK, tile_table, tile_rows, ws, kStaticScratchBytes,
+                           violations, stream);
 }
