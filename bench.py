@@ -3,7 +3,11 @@
 One step = one forward + backward of `MoMoE` (x, mask, s -> y; dy -> dx, dWl1, dWl2, ds)
 on the headline layer: B=4, S=2048 (8192 tokens), D=2048, H=1024, N=128 experts, K=8,
 bf16 with fp32 accumulation, save_percent=0.  Inputs are synthetic, seeded, and resident
-in HBM before the timed region.  Prints ONE JSON line.
+in HBM before the timed region.  Prints ONE JSON line: the headline figure from exactly
+`--steps` timed steps, and next to it the forward alone, the other save setting, a sustained
+figure from at least 2 s of back-to-back steps, the shader clock the GEMMs ran at, the layer
+with its router in front, per-kernel launch times with their fraction of the MFMA or HBM
+roofline, and the CPU oracle on the host cores.
 """
 import argparse
 import json
@@ -19,9 +23,12 @@ for _p in (ROOT, os.path.join(ROOT, "momoe-impl_amd"), os.path.join(ROOT, "tests
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command
 # (profiles/momoe_layer_headline_{fetch,write}_size.txt; fetch scaled x2.0, write x1.0 by the
-# 256 MiB copy in the same runs); None for a kernel that has not been measured.
+# 256 MiB copy in the same runs).  Counters cannot be read from inside this process, so these are
+# the figures of the profile run named in TRAFFIC_SOURCE, not of the run that prints them; None
+# for a kernel that has not been measured.
+TRAFFIC_SOURCE = "profiles/momoe_layer_headline_fetch_size.txt + _write_size.txt"
 MEASURED_TRAFFIC_BYTES = {
     "momoe_lin1_swiglu_fwd": 2 * 814482 * 1024 + 173802 * 1024,
     "momoe_lin1_swiglu_bwd": 2 * 924177 * 1024 + 398073 * 1024,
@@ -52,34 +59,54 @@ def kernel_flops(D, H, msum):
     }
 
 
-def cpu_baseline(D, H, N, K, budget_s=20.0):
-    """The oracle MoE layer (router restated in torch + per-expert loop + autograd backward)
-    on the host cores, on a reduced token count of the same layer."""
+def kernel_bytes(M, D, H, N, K):
+    """Algorithmic HBM bytes per launch of the bandwidth-bound kernels."""
+    msum = M * K
+    return {
+        # mask once, idx + inv (the reference's idx + which), cumsums, sizes
+        "momoe_index_build": N * M * 4 + 2 * msum * 4 + (N + 1) * 4 + N * 8,
+        "momoe_combine": msum * D * 2 + M * D * 2 + msum * 4,
+        "momoe_gs_scatter": msum * ((H + 127) // 128) * 4 + msum * 4 + msum * 4,
+        # bf16 logits in; mask, s, p_sel out (4 bytes each); Ng, Ks per token
+        "momoe_router_fwd": M * N * (2 + 12) + M * 8 + N * 4,
+        # G_s, p_sel, s, mask in (4 bytes each); bf16 logit gradient out
+        "momoe_router_bwd": M * N * (16 + 2) + M * 8,
+        # saved a|b and u in; gz, hs out; one partial sum per row
+        "momoe_swiglu_bwd_saved": msum * H * 2 * (2 + 1 + 2 + 1) + msum * 4,
+    }
+
+
+def cpu_baseline(D, H, N, K, budget_s=25.0):
+    """The oracle MoE layer as `MoE.forward` runs it (router -> per-expert loop -> bias update,
+    momoe/sample_moe.py:59-68) plus its autograd backward, in fp32 on the host cores, on a
+    reduced token count of the same layer."""
     import torch
     import oracle
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     Ms = 1024
-    x, W1, W2, mask, s, dy = headline_inputs(Ms, D, H, N, K, seed=1)
-    W1f, W2f = W1.float().requires_grad_(), W2.float().requires_grad_()
-    xf = x.bfloat16().float().requires_grad_()
-    sf = s.clone().requires_grad_()
+    x, W1, W2, _, _, dy = headline_inputs(Ms, D, H, N, K, seed=1)
+    Wg = torch.randn(D, N, generator=torch.Generator().manual_seed(2)) / D ** 0.5
+    moe = oracle.OracleMoE(D, H, N, K, 0, Wg_DN=Wg, Wl1_ND2H=W1.float(), Wl2_NHD=W2.float())
+    xf = x.bfloat16().float().reshape(1, Ms, D).requires_grad_()
+    dyf = dy.reshape(1, Ms, D)
     times = []
     t_start = time.time()
     for it in range(4):
         t0 = time.time()
-        y = oracle.experts_forward(xf, W1f, W2f, mask, sf)
-        y.backward(dy)
+        y = moe(xf)
+        y.backward(dyf)
         dt = time.time() - t0
-        W1f.grad = W2f.grad = xf.grad = sf.grad = None
+        moe.zero_grad(set_to_none=True)
+        xf.grad = None
         if it > 0:
             times.append(dt)
         if time.time() - t_start > budget_s and times:
             break
     best = min(times)
     return {"value": Ms / best, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"oracle MoE layer fwd+bwd, fp32, {Ms} of 8192 tokens of the headline layer "
-                      f"(D={D}, H={H}, N={N}, K={K}), best of {len(times)} runs, {best:.3f} s each"}
+            "sample": f"oracle MoE (router + experts + bias update) fwd+bwd, fp32, {Ms} of 8192 tokens of the "
+                      f"headline layer (D={D}, H={H}, N={N}, K={K}), best of {len(times)} runs, {best:.3f} s each"}
 
 
 def main():
@@ -152,35 +179,85 @@ def main():
     torch.cuda.synchronize()
     peak_extra_mib = (torch.cuda.max_memory_allocated() - base_mem) / 2**20
 
-    # per-kernel launch durations, HIP events on the launch stream, same region
+    # per-kernel launch durations (HIP events on the launch stream) and the shader clock the
+    # grouped GEMMs ran at (in-kernel counters), over `steps` more steps of the same loop
     per = {}
-    with _hip.kernel_timer() as kt:
+    with _hip.clock_trace() as ct, _hip.kernel_timer() as kt:
         for _ in range(args.steps):
             step(layer)
-    wcount = 0
-    for name, t in kt.durations_ms():
-        if name == "momoe_wgrad":
-            name = "momoe_wgrad[Wl2]" if wcount % 2 == 0 else "momoe_wgrad[Wl1]"
-            wcount += 1
-        per.setdefault(name, []).append(t)
-    # lin1 is launched twice per step at save_percent < 100 (forward, backward recomputation)
-    kernels = {k: {"launches_per_step": len(v) / args.steps, "avg_ms": sum(v) / len(v)} for k, v in per.items()}
+    clock_timed = ct.mhz()
+
+    def collect(kt, per):
+        wcount = 0
+        for name, t in kt.durations_ms():
+            if name == "momoe_wgrad":
+                name = "momoe_wgrad[Wl2]" if wcount % 2 == 0 else "momoe_wgrad[Wl1]"
+                wcount += 1
+            per.setdefault(name, []).append(t)
+
+    collect(kt, per)
+
+    # sustained rate: at least 2 s of back-to-back steps (the timed region above is a burst of
+    # a few tens of milliseconds, and these kernels run against the power limit)
+    n_sus = max(args.steps, int(2000.0 / ms) + 1)
+    with _hip.clock_trace() as ct:
+        ms_sustained = timed(layer, step, n_sus, 0)
+    clock_sustained = ct.mhz()
+
+    # the other save setting
+    other_sp = 100 if args.save_percent == 0 else 0
+    layer2 = make_layer(other_sp)
+    ms_other = timed(layer2, step, max(args.steps // 2, 3), 2)
+    if other_sp == 100:
+        with _hip.kernel_timer() as kt2:
+            for _ in range(3):
+                step(layer2)
+        for name, t in kt2.durations_ms():
+            if name == "momoe_swiglu_bwd_saved":
+                per.setdefault(name, []).append(t)
+    del layer2
+
+    # the layer with its router in front: MoE = TopKRouter -> MoMoE -> bias update
+    # (momoe/sample_moe.py:59-68), gate weights ~ N(0, 1/D)
+    Wg = torch.randn(D, N, generator=torch.Generator().manual_seed(3)) / D ** 0.5
+    moe = momoe_amd.MoE(D, H, N, K, 0, save_percent=args.save_percent, Wg_DN=Wg.to(dev),
+                        Wl1_ND2H=layer.Wl1_ND2H.data, Wl2_NHD=layer.Wl2_NHD.data)
+
+    def moe_step(m):
+        y = m(xd)
+        y.backward(dyd)
+        m.zero_grad(set_to_none=True)
+        xd.grad = None
+
+    ms_moe = timed(moe, moe_step, args.steps, 3)
+    with _hip.kernel_timer() as kt3:
+        for _ in range(args.steps):
+            moe_step(moe)
+    for name, t in kt3.durations_ms():
+        if name.startswith("momoe_router"):
+            per.setdefault(name, []).append(t)
+    del moe
+
+    launches = {k: len(v) / args.steps for k, v in per.items()}
+    launches["momoe_swiglu_bwd_saved"] = 1.0
+    kernels = {k: {"launches_per_step": launches[k], "avg_ms": sum(v) / len(v)} for k, v in per.items()}
     flops = kernel_flops(D, H, msum)
     for k, f in flops.items():
         if k in kernels:
             kernels[k]["tflops"] = f / kernels[k]["avg_ms"] / 1e9
             kernels[k]["frac_peak"] = kernels[k]["tflops"] / PEAK_BF16_TFLOPS
+    for k, b in kernel_bytes(M, D, H, N, K).items():
+        if k in kernels:
+            kernels[k]["algorithmic_bytes"] = b
+            kernels[k]["hbm_gbs"] = b / kernels[k]["avg_ms"] / 1e6
+            kernels[k]["frac_hbm_peak"] = kernels[k]["hbm_gbs"] / PEAK_HBM_GBS
     dom = max((k for k in kernels if k in flops),
               key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
     roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS,
-                "avg_launch_ms": kernels[dom]["avg_ms"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom)}
-
-    # the other save setting, and the layer with its router in front
-    other_sp = 100 if args.save_percent == 0 else 0
-    layer2 = make_layer(other_sp)
-    ms_other = timed(layer2, step, max(args.steps // 2, 3), 2)
-    del layer2
+                "avg_launch_ms": kernels[dom]["avg_ms"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                "traffic_source": TRAFFIC_SOURCE if dom in MEASURED_TRAFFIC_BYTES else None,
+                "shader_clock_mhz": clock_timed}
 
     useful = 18.0 * D * H * msum
     out = {
@@ -195,6 +272,10 @@ def main():
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": M / (ms_fwd * 1e-3),
         "fwd_tflops": 6.0 * D * H * msum / ms_fwd / 1e9,
         f"ms_per_step_save_percent_{other_sp}": ms_other,
+        "sustained_ms_per_step": ms_sustained, "sustained_steps": n_sus,
+        "sustained_tokens_per_s": M / (ms_sustained * 1e-3),
+        "shader_clock_mhz": clock_timed, "sustained_shader_clock_mhz": clock_sustained,
+        "ms_per_step_with_router": ms_moe, "tokens_per_s_with_router": M / (ms_moe * 1e-3),
         "peak_activation_mib": peak_extra_mib,
         "roofline": roofline, "kernels": kernels,
     }

@@ -43,6 +43,16 @@ extern "C" {
 int momoe_abi_version(void);
 const char* momoe_status_string(int status);
 
+/* Measurement aid, no counterpart in the reference.  ticks2: device pointer to two zeroed
+ * 64-bit counters, or NULL to stop.  While set, one wavefront of every grouped-GEMM launch
+ * (x.Wl1, h.Wl2, both data gradients, both weight gradients) adds the shader-clock ticks it ran
+ * for to ticks2[0] and the ticks of the constant 100 MHz counter over the same interval to
+ * ticks2[1]: 100 * ticks2[0] / ticks2[1] = average shader clock in MHz under those kernels.
+ * Process-wide setting, meant for a benchmark harness: launches in flight when it changes may
+ * use either value; the buffer must outlive every launch made while it is set.
+ */
+int momoe_set_clock_trace(unsigned long long* ticks2);
+
 /* ---- routing index -------------------------------------------------------
  * Replaces find_used_experts + scatter_cols_kernel (momoe/momoe.py:821-842,
  * 760-815) and the torch.sum at :830.
@@ -127,17 +137,27 @@ int momoe_combine(const void* rows_MsumD, const int32_t* inv_MK, void* out_MD,
  * momoe_dgrad_h:  u[r] = bf16( G_y[idx[r]] @ Wl2[i]^T )  (fp32 accumulate over D), the
  *   gradient of h before the gate weight; u_MsumH bf16 [Msum,H] in sorted order.
  *
- * momoe_lin1_swiglu_bwd, for the sorted rows r >= row_lo (those without saved a|b):
+ * momoe_lin1_swiglu_bwd, for the sorted rows without saved a|b:
  *   a|b  = x[idx[r]] @ Wl1[i]   (fp32, kept in registers)
  *   s    = s_NM[i, idx[r]],  sig = sigmoid(b)
  *   gz[r] = bf16( s u b sig | s u a sig (1 + b (1 - sig)) )       [G_a | G_b]
- *   hs[r] = bf16( s a b sig )       (h pre-scaled by the gate weight, for the Wl2 gradient)
+ *   hs    = bf16( s a b sig )       (h pre-scaled by the gate weight, for the Wl2 gradient)
  *   gs_part[p][r] = sum over the p-th block of MOMOE_GS_BLOCK hidden columns of u a b sig
  * (sum_p gs_part[p][r] = G_y[idx[r]] . (h[r] @ Wl2[i]) = dL/ds, by associativity).
  * gs_part fp32 [ceil(H/MOMOE_GS_BLOCK)][Msum].
+ * hs is written in the layout MOMOE_LAYOUT_TRANSPOSED of momoe_wgrad, zero padding included:
+ * hsT_GH32 bf16 [momoe_padded_rows(Msum, N) / 32][ld_hsT][32], ld_hsT >= H a multiple of 8.
  *
- * momoe_swiglu_bwd_saved, for the rows r < Msave: the same from the saved a|b (bf16); the whole
- * row sum goes to gs_part[0][r], zeros to the other parts.
+ * momoe_swiglu_bwd_saved: the same from the saved a|b (bf16) of the rows below Msave; the row
+ * sum is spread over the first ceil(H/256) parts, the other parts get zeros
+ * (nparts = ceil(H / MOMOE_GS_BLOCK)).
+ *
+ * Which of the two produces a row (the reference's own choice is per tile of its autotuned
+ * height, momoe/momoe.py:486): rows are taken in groups of 32 counted from their expert's first
+ * row; momoe_swiglu_bwd_saved produces the groups that lie entirely below Msave,
+ * momoe_lin1_swiglu_bwd (row_lo = Msave) all others, so that up to 31 rows just below Msave
+ * are recomputed although their a|b were saved.  Call both with the same Msave; either is a
+ * no-op when it has no rows (Msave = 0, row_lo = Msum).
  */
 int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32_t* idx_Msum,
                   const int32_t* tile_table, void* u_MsumH,
@@ -146,13 +166,15 @@ int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32_t* idx_Msu
 int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
                           const int32_t* tile_table, const void* u_MsumH,
                           const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
-                          int64_t row_lo, void* gz_Msum2H, void* hs_MsumH, float* gs_part,
+                          int64_t row_lo, void* gz_Msum2H, void* hsT_GH32, int64_t ld_hsT,
+                          float* gs_part,
                           int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
 
 int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH,
                            const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
                            const int32_t* idx_Msum, const int32_t* cumsums_N1, int64_t Msave,
-                           void* gz_Msum2H, void* hs_MsumH, float* gs_part, int64_t nparts,
+                           void* gz_Msum2H, void* hsT_GH32, int64_t ld_hsT,
+                           float* gs_part, int64_t nparts,
                            int64_t M, int64_t H, int64_t N, int64_t Msum, void* stream);
 
 /* momoe_gs_scatter: Gs_NM[i, idx[r]] = sum_p gs_part[p][r] for every sorted row r of
@@ -172,13 +194,25 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
                   void* stream);
 
 /* momoe_wgrad replaces weights_update_kernel (momoe/momoe.py:356-412):
- *   GW[i][x][y] = bf16( sum over sorted rows r of expert i of A[ra(r)][x] * B[rb(r)][y] )
- * with ra(r) = a_gather ? a_gather[r] : r (same for rb).  A bf16 with row stride lda
- * (>= X), B bf16 with row stride ldb (>= Y).  M = number of tokens (rows of a gathered
- * matrix, and the most rows an expert can hold); M * ld * 2 bytes must stay below 4 GiB.
- * Experts without rows get exact zeros.
- * Wl2 gradient: A = hs (X=H), B = G_y gathered by idx (Y=D).
- * Wl1 gradient: A = x gathered by idx (X=D), B = gz (Y=2H).
+ *   GW[i][x][y] = bf16( sum over sorted rows r of expert i of A(r, x) * B(r, y) ).
+ * Each operand comes in one of two layouts:
+ *   MOMOE_LAYOUT_ROWS        bf16 [row][feature] with row stride ld (>= features):
+ *                            A(r, x) = A[ra(r) * lda + x], ra(r) = a_gather ? a_gather[r] : r.
+ *   MOMOE_LAYOUT_TRANSPOSED  bf16 [padded sorted row / 32][ld][32] with ld >= features, no
+ *                            gather: the sorted row r of expert i (whose first sorted row is
+ *                            c = cumsums[i]) has the padded position
+ *                            p = ((c + 31) & ~31) + 32 * i + (r - c) < momoe_padded_rows(Msum, N),
+ *                            and its feature f sits at [(p / 32) * ld * 32 + f * 32 + p % 32];
+ *                            the positions between an expert's last row and the next multiple of
+ *                            32 must hold zeros.  This is how momoe_lin1_swiglu_bwd /
+ *                            momoe_swiglu_bwd_saved write hs: the contraction index is the fast
+ *                            one, which the kernel reads from LDS at twice the rate of the row
+ *                            layout, and each 32-row stage of a tile is one contiguous block.
+ *                            At most one operand may be transposed.
+ * M = number of tokens (rows of a gathered matrix, and the most rows an expert can hold);
+ * M * ld * 2 bytes (row layout) must stay below 4 GiB.  Experts without rows get exact zeros.
+ * Wl2 gradient: A = hs (transposed, X=H), B = G_y gathered by idx (Y=D).
+ * Wl1 gradient: A = x gathered by idx (X=D), B = gz (rows, Y=2H).
  * workspace: device scratch (16-byte aligned, contents undefined on entry and exit) for
  * fp32 partial tiles of MOMOE_WGRAD_PARTIAL_BYTES each.  An expert that holds many times
  * the average number of rows is contracted in several pieces so that its tiles do not
@@ -189,9 +223,12 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
  * summation order of a cut expert differs from that of an uncut one.
  */
 #define MOMOE_WGRAD_PARTIAL_BYTES 262144
+#define MOMOE_LAYOUT_ROWS 0
+#define MOMOE_LAYOUT_TRANSPOSED 1
+int64_t momoe_padded_rows(int64_t Msum, int64_t N);
 int64_t momoe_wgrad_workspace_bytes(int64_t N, int64_t X, int64_t Y, int64_t Msum);
-int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
-                const void* B_rows, int64_t ldb, const int32_t* b_gather,
+int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32_t* a_gather,
+                const void* B, int64_t ldb, int b_layout, const int32_t* b_gather,
                 const int32_t* cumsums_N1, void* GW_NXY,
                 int64_t M, int64_t N, int64_t X, int64_t Y, int64_t Msum,
                 void* workspace, int64_t workspace_bytes, void* stream);

@@ -26,9 +26,16 @@ constexpr int kWave = 64;
 //   first sorted row of that expert, number of rows of that expert}.
 constexpr int kTileHeader = 4;
 
+// Feature-major ("transposed") copies of sorted-row matrices, [feature][padded sorted row]: every
+// expert's rows start at a multiple of 32 and are followed by zeros up to the next multiple of
+// 32, so that a contraction over an expert's rows can read them in 32-row stages.  Padded
+// position of the first sorted row `row0` of expert `e` (momoe_padded_rows() bounds them all):
+__host__ __device__ __forceinline__ int padded_start(int row0, int e) { return ((row0 + 31) & ~31) + 32 * e; }
+
 struct TileCoord {
   int expert;  // expert index
   int row0;    // first sorted row of this tile
+  int prow0;   // padded position of that row
   int rows;    // valid rows in this tile (1..rows per tile)
   int tn;      // column block
   int mbase;   // first tile row owned by this wave (waves 0-3 / 4-7 split the tile's rows)
@@ -86,11 +93,12 @@ struct TileSched {
     TileCoord tc;
     tc.valid = r.any;
     if (!r.any) return tc;
-    // The expert's rows are cut into its nt row tiles of equal height (a multiple of 32),
-    // not into full tiles plus a remainder: tiles that share a weight block then take equally
-    // long and stay in step, and no tile streams a whole weight block for a handful of rows.
+    // The expert's rows are 32-row fragment rows, dealt to its nt row tiles as evenly as they
+    // go (the first few tiles hold one more), not full tiles plus a remainder: tiles that share
+    // a weight block then take nearly equally long and stay in step, no tile streams a whole
+    // weight block for a handful of rows, and only the expert's last fragment row is ragged.
     const int nt = (r.mi + bm - 1) / bm;
-    const int th = ((r.mi + nt - 1) / nt + 31) & ~31;
+    const int nfe = (r.mi + 31) >> 5, fbase = nfe / nt, fextra = nfe - fbase * nt;
     // Order inside an expert: bands of kBandTiles row tiles, each band crossing every column
     // block before the next band starts (row tile fastest inside a band).  The workgroups of
     // an XCD hold consecutive positions at any moment, so they share a few row tiles and a few
@@ -102,8 +110,10 @@ struct TileSched {
     const int tl = band * kBandTiles + in_band % band_rows;
     tc.tn = in_band / band_rows;
     tc.expert = r.expert;
-    tc.row0 = r.rstart + tl * th;
-    tc.rows = min(th, r.mi - tl * th);
+    const int f0 = tl * fbase + min(tl, fextra);  // first fragment row of this tile
+    tc.row0 = r.rstart + 32 * f0;
+    tc.prow0 = padded_start(r.rstart, r.expert) + 32 * f0;
+    tc.rows = min(32 * (fbase + (tl < fextra ? 1 : 0)), r.mi - 32 * f0);
     // the tile's fragment rows are dealt to the two wave rows as evenly as possible
     const int nf = (tc.rows + 31) >> 5, half = (nf + 1) >> 1;
     const bool upper = threadIdx.x >= 256;
@@ -132,6 +142,31 @@ __device__ __forceinline__ float bf2f(bf16 v) { return (float)v; }
 __device__ __forceinline__ bf16 f2bf(float v) { return (bf16)v; }
 
 __device__ __forceinline__ float sigmoidf_fast(float v) { return 1.0f / (1.0f + __expf(-v)); }
+
+// Measurement aid (momoe_set_clock_trace): while a trace buffer is set, one wavefront of every
+// grouped-GEMM launch adds the shader-clock ticks it ran for to buf[0] and the ticks of the
+// constant 100 MHz counter over the same interval to buf[1]; 100 * buf[0] / buf[1] is the
+// average shader clock in MHz while those kernels ran.
+unsigned long long* clock_trace_buffer();  // host side: the buffer in use, or nullptr
+struct ClockTrace {
+  unsigned long long* buf;
+  // start: subtract the counters, finish(): add them -- nothing is kept in registers in between
+  __device__ __forceinline__ explicit ClockTrace(unsigned long long* b) : buf(b) {
+    if (active()) {
+      atomicAdd(buf, 0ull - (unsigned long long)clock64());
+      atomicAdd(buf + 1, 0ull - (unsigned long long)wall_clock64());
+    }
+  }
+  __device__ __forceinline__ bool active() const {
+    return buf != nullptr && blockIdx.x == 0 && threadIdx.x == 0;
+  }
+  __device__ __forceinline__ void finish() const {
+    if (active()) {
+      atomicAdd(buf, (unsigned long long)clock64());
+      atomicAdd(buf + 1, (unsigned long long)wall_clock64());
+    }
+  }
+};
 
 inline int launch_status() {
   return hipGetLastError() == hipSuccess ? MOMOE_OK : MOMOE_ERR_LAUNCH;

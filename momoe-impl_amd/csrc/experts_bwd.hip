@@ -22,6 +22,7 @@ struct DhArgs {
   const int32_t* table;
   bf16* u;
   int D, H;
+  unsigned long long* clk;
 };
 
 // u = G_y[idx] . Wl2^T is an "NT" GEMM: both operands are k-contiguous (k = D).
@@ -67,16 +68,25 @@ struct DhProg {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
+  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.H + BN - 1) / BN);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   DhProg prog{p, p.D / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  trace.finish();
 }
 
-// SwiGLU backward for the sorted rows whose a|b were saved by the forward: one workgroup per
-// row, 8 hidden columns per thread and pass.
+// SwiGLU backward for the sorted rows whose a|b were saved by the forward.  One workgroup per
+// group of 32 padded sorted rows (an expert's rows start at a multiple of 32 in padded
+// positions, so a group never straddles two experts); it walks the hidden columns 64 at a time:
+// thread t holds row t/8 and 8 of the 64 columns, writes its piece of gz row-major, and passes
+// its piece of hs through LDS transposed, from where 8 consecutive rows of one column leave per
+// thread for the transposed copy of hs.  Rows of the group past the expert's last one become the zero padding.
+// A group belongs to this kernel when all of its rows lie below `Msave`; the remaining groups
+// (those of the expert that Msave cuts, from the group holding Msave on, and all later experts)
+// are produced by momoe_lin1_swiglu_bwd, which applies the same rule.
 struct SavedArgs {
   const bf16* ab;
   const bf16* u;
@@ -85,67 +95,91 @@ struct SavedArgs {
   const int32_t* idx;
   const int32_t* cumsums;
   bf16* gz;
-  bf16* hs;
+  bf16* hst;
+  int64_t ldt;
   float* gs_part;
   int nparts;
-  int64_t msum;
+  int64_t msum, msave;
   int H, N, M;
 };
 
+constexpr int kSavedCols = 64;    // hidden columns per pass
+constexpr int kSavedSpan = 256;   // hidden columns per workgroup: blockIdx.y selects the span
+static_assert(kSavedSpan % MOMOE_GS_BLOCK == 0 && kSavedSpan % kSavedCols == 0, "spans cover whole parts");
+
 __global__ __launch_bounds__(256) void swiglu_bwd_saved_kernel(SavedArgs p) {
-  const int64_t r = blockIdx.x;
-  const int H = p.H;
-  __shared__ float s_red[4];
-  if (r >= p.cumsums[p.N]) {
-    // The routing holds fewer pairs than M*K (a token with fewer than K experts): this sorted
-    // row does not exist and its token id was never written.  Its outputs are defined zeros.
-    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
-      *(bf16x8*)(p.gz + r * 2 * H + c) = z;
-      *(bf16x8*)(p.gz + r * 2 * H + H + c) = z;
-      *(bf16x8*)(p.hs + r * H + c) = z;
-    }
-    for (int q = threadIdx.x; q < p.nparts; q += 256) p.gs_part[(int64_t)q * p.msum + r] = 0.0f;
-    return;
-  }
-  // expert of row r: the i with cumsums[i] <= r < cumsums[i+1]
-  int lo = 0, hi = p.N;
+  __shared__ __attribute__((aligned(16))) bf16 tr[2][kSavedCols * 32];  // [pass parity][column][row]
+  const int H = p.H, N = p.N;
+  const int pg = blockIdx.x * 32;  // first padded position of the group
+  // expert whose padded range holds pg: the last e with padded_start(cumsums[e], e) <= pg
+  int lo = 0, hi = N;
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
-    if (p.cumsums[mid] <= r) lo = mid; else hi = mid;
+    if (padded_start(min(p.cumsums[mid], (int)p.msum), mid) <= pg) lo = mid; else hi = mid;
   }
+  const int c0 = min(p.cumsums[lo], (int)p.msum), c1 = min(p.cumsums[lo + 1], (int)p.msum);
+  const int local = pg - padded_start(c0, lo);  // rows of the expert before this group
+  const int valid = min(32, c1 - c0 - local);   // rows of the group that exist
+  if (local < 0 || valid <= 0) return;           // padding between two experts
+  const int64_t r0 = (int64_t)c0 + local;        // first sorted row of the group
+  if (r0 + valid > p.msave) return;              // not (entirely) below the save boundary
+
+  const int t = threadIdx.x, row = t >> 3, cc = (t & 7) * 8;
+  const bool rowok = row < valid;
+  const int64_t r = r0 + min(row, valid - 1);
   const int tok = min(max(p.idx[r], 0), p.M - 1);
   const float sv = p.s[(int64_t)lo * p.ssn + (int64_t)tok * p.ssm];
   const bf16* a_row = p.ab + r * 2 * H;
   const bf16* u_row = p.u + r * H;
   float gsum = 0.0f;
-  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
-    const bf16x8 a8 = *(const bf16x8*)(a_row + c);
-    const bf16x8 b8 = *(const bf16x8*)(a_row + H + c);
-    const bf16x8 u8 = *(const bf16x8*)(u_row + c);
-    bf16x8 ga, gb, hv;
+  int par = 0;
+  const int hbeg = blockIdx.y * kSavedSpan, hend = min(H, hbeg + kSavedSpan);
+  for (int h0 = hbeg; h0 < hend; h0 += kSavedCols, par ^= 1) {
+    const int c = h0 + cc;
+    bf16x8 hv = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (c < H) {
+      const bf16x8 a8 = *(const bf16x8*)(a_row + c);
+      const bf16x8 b8 = *(const bf16x8*)(a_row + H + c);
+      const bf16x8 u8 = *(const bf16x8*)(u_row + c);
+      bf16x8 ga, gb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float a = (float)a8[e], b = (float)b8[e], u = (float)u8[e];
+        const float sg = sigmoidf_fast(b);
+        const float hval = a * b * sg;
+        gsum += u * hval;
+        const float gh = sv * u;
+        ga[e] = (bf16)(gh * b * sg);
+        gb[e] = (bf16)(gh * a * sg * (1.0f + b * (1.0f - sg)));
+        hv[e] = (bf16)(rowok ? sv * hval : 0.0f);
+      }
+      if (rowok) {
+        *(bf16x8*)(p.gz + r * 2 * H + c) = ga;
+        *(bf16x8*)(p.gz + r * 2 * H + H + c) = gb;
+      }
+    }
+    // transposed staging: column-major, the four 8-row groups of a column rotated by the
+    // column so that the 8 threads of a row (columns 8 apart) do not share a bank
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float a = (float)a8[e], b = (float)b8[e], u = (float)u8[e];
-      const float sg = sigmoidf_fast(b);
-      const float hval = a * b * sg;
-      gsum += u * hval;
-      const float gh = sv * u;
-      ga[e] = (bf16)(gh * b * sg);
-      gb[e] = (bf16)(gh * a * sg * (1.0f + b * (1.0f - sg)));
-      hv[e] = (bf16)(sv * hval);
+      const int col = cc + e;
+      tr[par][col * 32 + (((row >> 3) ^ (col >> 3)) & 3) * 8 + (row & 7)] = hv[e];
     }
-    *(bf16x8*)(p.gz + r * 2 * H + c) = ga;
-    *(bf16x8*)(p.gz + r * 2 * H + H + c) = gb;
-    *(bf16x8*)(p.hs + r * H + c) = hv;
+    __syncthreads();  // one barrier per pass: the other buffer is rewritten only after the next one
+    const int col = t >> 2, rg = t & 3;
+    if (h0 + col < H) {
+      const bf16x8 v = *(const bf16x8*)(&tr[par][col * 32 + ((rg ^ (col >> 3)) & 3) * 8]);
+      *(bf16x8*)(p.hst + ((int64_t)blockIdx.x * p.ldt + h0 + col) * 32 + rg * 8) = v;
+    }
   }
+  // dL/ds of the row: the 8 threads of a row are consecutive lanes
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) gsum += __shfl_xor(gsum, o);
-  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = gsum;
-  __syncthreads();
-  if (threadIdx.x == 0) p.gs_part[r] = s_red[0] + s_red[1] + s_red[2] + s_red[3];
-  // the whole row sum sits in part 0
-  for (int q = 1 + threadIdx.x; q < p.nparts; q += 256) p.gs_part[(int64_t)q * p.msum + r] = 0.0f;
+  for (int o = 4; o > 0; o >>= 1) gsum += __shfl_xor(gsum, o);
+  // the sum over this workgroup's span goes to part blockIdx.y; the parts that no span owns
+  // (there are ceil(H/128) parts and ceil(H/256) spans) are zeroed by the first span
+  if (rowok && (t & 7) == 0) p.gs_part[(int64_t)blockIdx.y * p.msum + r] = gsum;
+  if (blockIdx.y == 0 && rowok)
+    for (int q = gridDim.y + (t & 7); q < p.nparts; q += 8) p.gs_part[(int64_t)q * p.msum + r] = 0.0f;
 }
 
 struct DxArgs {
@@ -154,6 +188,7 @@ struct DxArgs {
   const int32_t* table;
   bf16* gxs;
   int D, H;
+  unsigned long long* clk;
 };
 
 // gxs = gz . Wl1^T: contraction over the 2H contiguous columns of both operands.
@@ -194,12 +229,14 @@ struct DxProg {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
+  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   DxProg prog{p, (2 * p.H) / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  trace.finish();
 }
 
 __global__ __launch_bounds__(256) void gs_scatter_kernel(const float* __restrict__ part, int nparts,
@@ -244,7 +281,7 @@ extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
   DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, idx_Msum, tile_table, (bf16*)u_MsumH, (int)D,
-           (int)H};
+           (int)H, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(dgrad_h_kernel, kBwdLds, once);
   dgrad_h_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
@@ -254,23 +291,27 @@ extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32
 extern "C" int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH, const float* s_NM,
                                       int64_t s_stride_n, int64_t s_stride_m,
                                       const int32_t* idx_Msum, const int32_t* cumsums_N1,
-                                      int64_t Msave, void* gz_Msum2H, void* hs_MsumH,
-                                      float* gs_part, int64_t nparts, int64_t M, int64_t H,
-                                      int64_t N, int64_t Msum, void* stream) {
-  if (!ab_save || !u_MsumH || !s_NM || !idx_Msum || !cumsums_N1 || !gz_Msum2H || !hs_MsumH ||
+                                      int64_t Msave, void* gz_Msum2H, void* hsT_GH32,
+                                      int64_t ld_hsT, float* gs_part, int64_t nparts, int64_t M,
+                                      int64_t H, int64_t N, int64_t Msum, void* stream) {
+  if (!ab_save || !u_MsumH || !s_NM || !idx_Msum || !cumsums_N1 || !gz_Msum2H || !hsT_GH32 ||
       !gs_part)
     return MOMOE_ERR_BAD_ARG;
   if (Msave < 0 || Msave > Msum || nparts <= 0 || M <= 0 || H <= 0 || N <= 0 || Msum <= 0)
     return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_Msum2H) || !aligned16(hs_MsumH))
+  if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_Msum2H) || !aligned16(hsT_GH32))
     return MOMOE_ERR_BAD_ARG;
-  if (H % 8 != 0 || Msum >= (1ll << 31) || M >= (1ll << 31) || nparts > (1 << 20))
+  const int64_t mpad = momoe_padded_rows(Msum, N);
+  if (ld_hsT < H || ld_hsT % 8 != 0) return MOMOE_ERR_BAD_ARG;
+  if (H % 8 != 0 || mpad >= (1ll << 31) || M >= (1ll << 31) || nparts > (1 << 20))
     return MOMOE_ERR_UNSUPPORTED;
   if (Msave == 0) return MOMOE_OK;
   SavedArgs a{(const bf16*)ab_save, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m, idx_Msum,
-              cumsums_N1, (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part, (int)nparts, Msum, (int)H,
-              (int)N, (int)M};
-  swiglu_bwd_saved_kernel<<<(unsigned)Msave, 256, 0, (hipStream_t)stream>>>(a);
+              cumsums_N1, (bf16*)gz_Msum2H, (bf16*)hsT_GH32, ld_hsT, gs_part, (int)nparts, Msum,
+              Msave, (int)H, (int)N, (int)M};
+  const int64_t spans = cdiv64(H, kSavedSpan);
+  if (spans > nparts || spans > 65535) return MOMOE_ERR_BAD_ARG;  // nparts = ceil(H / MOMOE_GS_BLOCK)
+  swiglu_bwd_saved_kernel<<<dim3((unsigned)(mpad / 32), (unsigned)spans), 256, 0, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -294,7 +335,7 @@ extern "C" int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H,
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
   DxArgs a{(const bf16*)gz_Msum2H, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
-           (int)H};
+           (int)H, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(dgrad_x_kernel, kBwdLds, once);
   dgrad_x_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);

@@ -27,9 +27,11 @@ struct Lin1Args {
   const float* s;
   int64_t ssn, ssm;
   bf16* gz;
-  bf16* hs;
+  bf16* hst;    // hs in groups of 32 padded sorted rows, [group][ldt features][32]
+  int64_t ldt;
   float* gs_part;
   int64_t msum;
+  unsigned long long* clk;
 };
 
 // Tile = 256 rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
@@ -135,6 +137,10 @@ struct Lin1Prog {
       for (int q = 0; q < 4; ++q) uq[q] = *(const bf16x4*)(p.u + r * H + min(j0 + acc_col(q), H - 4));
     };
     RowStager<1> stager1(epi, 1);
+    // Rows below the save boundary are not this kernel's: the boundary is moved down to a
+    // multiple of 32 rows from the expert's first row (tiles start at such multiples), so that
+    // a whole 32-row fragment row is either produced here or by momoe_swiglu_bwd_saved.
+    const int rl_lo = p.ab_lo > tc.row0 ? (int)((p.ab_lo - tc.row0) & ~(int64_t)31) : 0;
     float gsums[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -163,22 +169,45 @@ struct Lin1Prog {
         stager.put(0, q, pack_bf16x4(va[0], va[1], va[2], va[3]));
         stager1.put(0, q, pack_bf16x4(vb[0], vb[1], vb[2], vb[3]));
       }
+      const int rl0 = tc.mbase + 32 * i;  // first tile row of this fragment row
+      const bool mine = rl0 >= rl_lo;      // wave-uniform
       auto dst = [&](bf16* mat, int64_t ld, int col0) {
         return [=, *this](int row, int col) -> bf16* {
-          const int rl = (tc.mbase + 32 * i) + row;
-          const int64_t r = (int64_t)tc.row0 + rl;
-          if (rl >= tc.rows || j0 + col >= H || r < p.ab_lo) return nullptr;
-          return mat + r * ld + col0 + j0 + col;
+          const int rl = rl0 + row;
+          if (rl >= tc.rows || j0 + col >= H || !mine) return nullptr;
+          return mat + ((int64_t)tc.row0 + rl) * ld + col0 + j0 + col;
         };
       };
       stager.flush(dst(p.gz, 2 * H, 0));
       stager1.flush(dst(p.gz, 2 * H, H));
+      // hs^T: the 32 x 32 fragment goes through the staging area transposed ([column][row],
+      // the four 8-row groups of a column permuted so that the two half-waves, which write
+      // columns 4 apart, use different banks) and leaves it as 8 consecutive rows of one column
+      // per lane.  Rows past the expert's last one are written as zeros: they are the padding
+      // the weight-gradient GEMM reads.
+      {
+        bf16* tst = stager.st;
+        const int row = acc_row();
+        const bool rowok = rl0 + row < tc.rows;
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        stager.put(0, q, pack_bf16x4(acc[0][i][4 * q], acc[0][i][4 * q + 1], acc[0][i][4 * q + 2],
-                                     acc[0][i][4 * q + 3]));
-      stager.flush(dst(p.hs, H, 0));
-      gsums[i] = (tc.mbase + 32 * i) + acc_row() < tc.rows ? gsum : 0.0f;
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int col = acc_col(q) + e;
+            const int grp = (row >> 3) ^ ((col >> 2) & 3);
+            tst[col * 32 + grp * 8 + (row & 7)] = (bf16)(rowok ? acc[0][i][4 * q + e] : 0.0f);
+          }
+        const int l = threadIdx.x & 63;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+          const int col = pass * 16 + (l >> 2), rg = l & 3;
+          const bf16x8 v = *(const bf16x8*)(tst + col * 32 + ((rg ^ ((col >> 2) & 3)) * 8));
+          // the fragment's 32 columns x 32 rows are 2 KiB of consecutive memory
+          if (mine && j0 + col < H)
+            *(bf16x8*)(p.hst + ((int64_t)((tc.prow0 + rl0) >> 5) * p.ldt + j0 + col) * 32 + rg * 8) = v;
+        }
+      }
+      gsums[i] = rl0 + acc_row() < tc.rows ? gsum : 0.0f;
     }
     // every wave is done with its staging area before the row sums overwrite it
     wait_lgkm0();
@@ -191,7 +220,7 @@ struct Lin1Prog {
     }
     wait_lgkm0();  // the row sums are in LDS (a full fence would also wait for the stores above)
     __builtin_amdgcn_s_barrier();
-    if ((int)threadIdx.x < tc.rows && (int64_t)tc.row0 + threadIdx.x >= p.ab_lo)
+    if ((int)threadIdx.x < tc.rows && (int)threadIdx.x >= rl_lo)
       p.gs_part[(int64_t)tc.tn * p.msum + tc.row0 + threadIdx.x] =
           red[threadIdx.x] + red[BM + threadIdx.x] + red[2 * BM + threadIdx.x] +
           red[3 * BM + threadIdx.x];
@@ -203,6 +232,7 @@ struct Lin1Prog {
 template <bool BWD>
 __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   using Prog = Lin1Prog<BWD>;
+  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   // without an h output only rows >= ab_lo are wanted: experts entirely below are skipped
   const int first_tile =
@@ -212,6 +242,7 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
   Prog prog{p, p.D / kBK, wn, dyn_lds() + kStages * Ring::STAGE};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  trace.finish();
 }
 
 struct Lin2Args {
@@ -223,6 +254,7 @@ struct Lin2Args {
   const int32_t* table;
   bf16* ys;
   int D, H;
+  unsigned long long* clk;
 };
 
 struct Lin2Prog {
@@ -272,12 +304,14 @@ struct Lin2Prog {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
+  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   Lin2Prog prog{p, p.H / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  trace.finish();
 }
 
 // out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.
@@ -332,7 +366,7 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   if (st != MOMOE_OK) return st;
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
-             nullptr, nullptr, 0, 0, nullptr, nullptr, nullptr, Msum};
+             nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, Msum, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(lin1_swiglu_kernel<false>, kFwdLds, once);
   lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
@@ -343,21 +377,22 @@ extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
                                      const int32_t* idx_Msum, const int32_t* tile_table,
                                      const void* u_MsumH, const float* s_NM, int64_t s_stride_n,
                                      int64_t s_stride_m, int64_t row_lo, void* gz_Msum2H,
-                                     void* hs_MsumH, float* gs_part, int64_t M, int64_t D,
-                                     int64_t H, int64_t N, int64_t Msum, void* stream) {
+                                     void* hsT_GH32, int64_t ld_hsT, float* gs_part, int64_t M,
+                                     int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream) {
   if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || !u_MsumH || !s_NM || !gz_Msum2H ||
-      !hs_MsumH || !gs_part)
+      !hsT_GH32 || !gs_part)
     return MOMOE_ERR_BAD_ARG;
   if (row_lo < 0 || row_lo > Msum) return MOMOE_ERR_BAD_ARG;
   if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)u_MsumH & 7) ||
-      !aligned16(gz_Msum2H) || !aligned16(hs_MsumH))
+      !aligned16(gz_Msum2H) || !aligned16(hsT_GH32))
     return MOMOE_ERR_BAD_ARG;
+  if (ld_hsT < H || ld_hsT % 8 != 0) return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
   if (row_lo == Msum) return MOMOE_OK;
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, nullptr, nullptr,
              row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
-             (bf16*)gz_Msum2H, (bf16*)hs_MsumH, gs_part, Msum};
+             (bf16*)gz_Msum2H, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(lin1_swiglu_kernel<true>, kFwdLds, once);
   lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
@@ -376,7 +411,7 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, co
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
   Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
-             idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H};
+             idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(lin2_scale_kernel, kFwdLds, once);
   lin2_scale_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);

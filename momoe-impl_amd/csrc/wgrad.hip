@@ -1,8 +1,17 @@
 // Weight-gradient grouped GEMM: GW[i] = A_i^T . B_i, contracting over the sorted
-// rows of expert i.  Both operands are stored [row][feature], i.e. k-strided, so
-// both go through the LDS transpose read.  Rows may be gathered through an index
-// (x and G_y are never materialised in sorted order); the k-values past the expert's
-// last row are zeroed in registers.
+// rows of expert i.  An operand is handed over in one of two layouts:
+//   rows        [row][feature] (optionally gathered through an index: x and G_y are never
+//               materialised in sorted order).  The contraction index is the slow one, so its
+//               fragments come through the LDS transpose read, at half the rate of a plain read.
+//   transposed  [padded sorted row / 32][feature][32]: the producing kernel wrote the matrix in
+//               groups of 32 rows, feature-major inside a group (hs), each expert's rows starting
+//               at a multiple of 32 and zero-filled up to the next multiple of 32.  The
+//               contraction index is the fast one: plain 16-byte fragment reads, and a stage is
+//               one contiguous 16 KiB block in memory.
+// Per wave and k-step the 4-fragment side of the 128 x 64 wave tile reads twice the LDS bytes of
+// the 2-fragment side, so the transposed operand is given the 4 fragments: it is the M side
+// (FM=4, FN=2) when A is transposed and the N side (FM=2, FN=4) when B is.
+// The k-values past the expert's last row are zeroed in registers on the M side.
 #include <algorithm>
 
 #include "gemm_tile.hpp"
@@ -12,15 +21,51 @@ namespace {
 
 constexpr int BX = 256;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
-constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 x 64
-using Ring = StageRing<TGatherDma, TGatherDma>;
-constexpr size_t kWgradLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+constexpr int kRingBytes = kStages * 2 * TLayout::LDS_ELEMS * 2;  // every operand kind: 16 KiB per stage
+constexpr size_t kWgradLds = kRingBytes + kEpilogueLds;  // stage ring + per-wave store staging
 constexpr int kMaxWgradExperts = 4096;  // 20 bytes of prefix sums per expert fit the stage ring
 constexpr int kMaxWorkgroups = 256;       // the workspace query assumes no more persistent workgroups
 constexpr int kSplitsPerWorkgroup = 8;  // large experts are cut into pieces of 1/8 .. 1/4 of a
                                         // workgroup's share of the launch
 static_assert(BX * BY * 4 == MOMOE_WGRAD_PARTIAL_BYTES, "size of one fp32 partial tile");
-static_assert((size_t)(kMaxWgradExperts + 1) * 20 + 512 <= Ring::BYTES, "prefix sums overlay the ring");
+static_assert((size_t)(kMaxWgradExperts + 1) * 20 + 512 <= kRingBytes, "prefix sums overlay the ring");
+
+// "rows" operand of a work item: the gathered / sorted rows [rb, re)
+struct RowsOperand : TGatherDma {
+  __device__ __forceinline__ void begin_piece(const int32_t* gather_, int64_t ld_, int rb, int re, int) {
+    set_rows(gather_, ld_, rb, re);
+  }
+};
+// "transposed" operand: groups of 32 padded sorted rows, feature-major inside a group: feature f
+// of padded sorted row p at mat[(p / 32) * ld * 32 + f * 32 + p % 32], ld >= number of features.
+// The 256 features x 32 rows of one stage are 16 KiB of consecutive memory.
+struct TransposedOperand {
+  using R = RDma<256>;
+  static constexpr int NCH = R::NCH;
+  static constexpr int LDS_ELEMS = R::LDS_ELEMS;
+  static_assert(LDS_ELEMS == TLayout::LDS_ELEMS, "same stage size as the other operand kind");
+  R r;
+  int64_t gstride;  // elements between consecutive 32-row groups
+  int g0;           // group of the first row of the piece
+  __device__ __forceinline__ void begin_piece(const int32_t*, int64_t ld_, int, int, int prow) {
+    gstride = ld_ * 32;
+    g0 = prow >> 5;
+  }
+  // features [f0, f0+256) of the matrix; features >= nfeat are clamped to the last one
+  __device__ __forceinline__ void set_cols(const bf16* mat, int f0, int nfeat) {
+    r.init(mat + (int64_t)g0 * gstride + (int64_t)f0 * 32,
+           [&](int row, int) { return (uint32_t)min(row, nfeat - 1 - f0) * 64u; });
+  }
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+    const int w = threadIdx.x >> 6;
+    const bf16* b = r.base + (int64_t)kt * gstride;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) dma16(b, r.off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
+  }
+  template <int S>
+  __device__ __forceinline__ void issue_head(uint32_t stage) { issue(S, stage); }
+  static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) { return R::frag(stage, c0, kk); }
+};
 
 struct WgradArgs {
   const bf16* a;
@@ -36,13 +81,30 @@ struct WgradArgs {
   int N, X, Y;
   int tiles_x, tiles_y;
   int msum;       // rows of the sorted matrices: row counts are clamped to it
+  unsigned long long* clk;
 };
 
 struct WTile {
   int expert, x0, y0;
   int rb, re;  // sorted rows this work item contracts over
+  int prow;    // padded position of row rb (transposed operands)
   int slot;    // partial tile to write, or -1: the item covers the whole expert and stores bf16
   bool valid;
+};
+
+// How the 8 waves share the 256 x 256 output tile: FM x FN fragments of 32 x 32 per wave.
+template <int FM, int FN>
+struct WaveTile {
+  static_assert(FM * FN == 8 && (FM == 4 || FM == 2), "128 x 64 or 64 x 128 per wave");
+  static constexpr int WAVES_N = 256 / (32 * FN);  // waves side by side
+  int m_org[FM], n_org[FN];
+  __device__ __forceinline__ WaveTile() {
+    const int wave = threadIdx.x >> 6, wm = wave / WAVES_N, wn = wave % WAVES_N;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) m_org[i] = wm * (32 * FM) + 32 * i;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) n_org[j] = wn * (32 * FN) + 32 * j;
+  }
 };
 
 constexpr int kEpilogueCost = 4;  // a tile's epilogue, in units of one k-stage of its main loop
@@ -170,25 +232,29 @@ __device__ __forceinline__ Plan build_cost_plan(const WgradArgs& p, int tpe) {
 }
 
 // bf16 store of one output tile from the accumulators (non-temporal: a weight gradient is
-// not read again by this kernel)
+// not read again by this kernel); two fragments (64 columns) go through the staging area at a time
+template <int FM, int FN>
 __device__ __forceinline__ void store_gw_tile(const WgradArgs& p, RowStager<2>& stager,
                                               f32x16 (&acc)[FN][FM], int expert, int x0, int y0t,
-                                              const int (&m_org)[FM], int wn) {
+                                              const WaveTile<FM, FN>& wt) {
   bf16* out = p.gw + (int64_t)expert * p.X * p.Y;
-  const int y0 = y0t + wn * 64;  // first output column of this wave
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
 #pragma unroll
-    for (int f = 0; f < FN; ++f)
+    for (int f0 = 0; f0 < FN; f0 += 2) {
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd)
-        stager.put(f, qd, pack_bf16x4(acc[f][i][4 * qd], acc[f][i][4 * qd + 1],
-                                      acc[f][i][4 * qd + 2], acc[f][i][4 * qd + 3]));
-    stager.flush<true>([&](int row, int col) -> bf16* {
-      const int x = x0 + m_org[i] + row;
-      if (x >= p.X || y0 + col >= p.Y) return nullptr;
-      return out + (int64_t)x * p.Y + y0 + col;
-    });
+      for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd)
+          stager.put(f, qd, pack_bf16x4(acc[f0 + f][i][4 * qd], acc[f0 + f][i][4 * qd + 1],
+                                        acc[f0 + f][i][4 * qd + 2], acc[f0 + f][i][4 * qd + 3]));
+      const int y0 = y0t + wt.n_org[f0];  // first output column of these two fragments
+      stager.flush<true>([&](int row, int col) -> bf16* {
+        const int x = x0 + wt.m_org[i] + row;
+        if (x >= p.X || y0 + col >= p.Y) return nullptr;
+        return out + (int64_t)x * p.Y + y0 + col;
+      });
+    }
   }
 }
 
@@ -196,6 +262,7 @@ __device__ __forceinline__ void store_gw_tile(const WgradArgs& p, RowStager<2>& 
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // A partial tile is kept in accumulator order: per wave, per fragment, 4 x (64 lanes x 16 B).
+template <int FM, int FN>
 __device__ __forceinline__ f32x4* partial_piece(float* ws, int slot, int i, int f, int qd) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   return (f32x4*)(ws + (int64_t)slot * (BX * BY)) +
@@ -212,8 +279,11 @@ __device__ __forceinline__ f32x4* partial_piece(float* ws, int slot, int i, int 
 // them up.
 // CUT = false is the launch in which no expert can reach the cutting length (the host knows:
 // an expert holds at most M rows): the bookkeeping of pieces is compiled out.
-template <bool CUT>
+template <bool CUT, class AOp, class BOp, int FM, int FN>
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
+  using Ring = StageRing<AOp, BOp>;
+  static_assert(Ring::BYTES == kRingBytes, "ring size assumed by the launch");
+  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   const int tpe = p.tiles_x * p.tiles_y;
   const int xcd = blockIdx.x & 7, stride = gridDim.x >> 3;
@@ -270,6 +340,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
       t.y0 = (q % p.tiles_y) * BY;
       t.rb = min(load_uniform(p.cumsums + expert), p.msum);
       t.re = min(load_uniform(p.cumsums + expert + 1), p.msum);
+      t.prow = padded_start(t.rb, expert);
       t.slot = -1;
       return t;
     }
@@ -289,10 +360,12 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     t.y0 = (q % p.tiles_y) * BY;
     t.rb = min(ex_re, ex_rb + piece * ep.chunk * kBK);
     t.re = min(ex_re, t.rb + ep.chunk * kBK);
+    t.prow = padded_start(ex_rb, ex) + (t.rb - ex_rb);
     t.slot = ep.splits > 1 ? ex_slot + it : -1;
     return t;
   };
-  TGatherDma A, B;
+  AOp A;
+  BOp B;
   int cur_rb = -1, cur_re = -1;
   // the rows of a piece (and the ids of the first of them) are looked up when the workgroup
   // moves on to a new piece; every tile of the piece then reuses them
@@ -301,20 +374,21 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     if (t.rb != cur_rb || t.re != cur_re) {
       cur_rb = t.rb;
       cur_re = t.re;
-      A.set_rows(p.ga, p.lda, t.rb, t.re);
-      B.set_rows(p.gb, p.ldb, t.rb, t.re);
+      A.begin_piece(p.ga, p.lda, t.rb, t.re, t.prow);
+      B.begin_piece(p.gb, p.ldb, t.rb, t.re, t.prow);
     }
     A.set_cols(p.a, t.x0, p.X);
     B.set_cols(p.b, t.y0, p.Y);
     gemm_issue_first(A, B, ring, (t.re - t.rb + kBK - 1) / kBK);
   };
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  const int n_org[FN] = {wn * 64, wn * 64 + 32};
+  const WaveTile<FM, FN> wt;
   RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
 
   WTile tc = next_tile();
-  if (!tc.valid) return;
+  if (!tc.valid) {
+    trace.finish();
+    return;
+  }
   start(tc);
   while (true) {
     f32x16 acc[FN][FM];
@@ -323,11 +397,11 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     const int ktail = tc.re - tc.rb - (ktiles - 1) * kBK;
     const WTile nx = next_tile();
     if (ktiles > 0)
-      gemm_mainloop<TGatherDma, TGatherDma, FM, FN, FM>(A, B, acc, ktiles, ring, m_org, n_org, [] {}, ktail);
+      gemm_mainloop<AOp, BOp, FM, FN, FM>(A, B, acc, ktiles, ring, wt.m_org, wt.n_org, [] {}, ktail);
     if (nx.valid) start(nx);
 
     if (!CUT || tc.slot < 0) {
-      store_gw_tile(p, stager, acc, tc.expert, tc.x0, tc.y0, m_org, wn);
+      store_gw_tile<FM, FN>(p, stager, acc, tc.expert, tc.x0, tc.y0, wt);
     } else {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
@@ -337,23 +411,24 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
           for (int qd = 0; qd < 4; ++qd) {
             f32x4 v = {acc[f][i][4 * qd], acc[f][i][4 * qd + 1], acc[f][i][4 * qd + 2],
                        acc[f][i][4 * qd + 3]};
-            *partial_piece(p.ws, tc.slot, i, f, qd) = v;
+            *partial_piece<FM, FN>(p.ws, tc.slot, i, f, qd) = v;
           }
     }
     if (!nx.valid) break;
     tc = nx;
   }
+  trace.finish();
 }
 
 // Adds up the partial tiles of the experts that wgrad_kernel cut into pieces and stores the
 // bf16 result; one workgroup per output tile, same register layout as the GEMM.
+template <int FM, int FN>
 __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(WgradArgs p) {
   const int tpe = p.tiles_x * p.tiles_y;
   const Plan pl = build_plan(p, tpe);
   const int ncut = pl.ctiles[p.N];
-  const int wave = threadIdx.x >> 6, wm = wave >> 2, wn = wave & 3;
-  const int m_org[FM] = {wm * 128, wm * 128 + 32, wm * 128 + 64, wm * 128 + 96};
-  RowStager<2> stager(dyn_lds() + kStages * Ring::STAGE);
+  const WaveTile<FM, FN> wt;
+  RowStager<2> stager((bf16*)((char*)dyn_lds() + kRingBytes));
   for (int t = blockIdx.x; t < ncut; t += gridDim.x) {
     int lo = 0, hi = p.N;  // ctiles[lo] <= t < ctiles[hi]; the last such lo is the cut expert
     while (hi - lo > 1) {
@@ -372,12 +447,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(WgradArgs p) {
         for (int f = 0; f < FN; ++f)
 #pragma unroll
           for (int qd = 0; qd < 4; ++qd) {
-            const f32x4 v = *partial_piece(p.ws, slot, i, f, qd);
+            const f32x4 v = *partial_piece<FM, FN>(p.ws, slot, i, f, qd);
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[f][i][4 * qd + r] += v[r];
           }
     }
-    store_gw_tile(p, stager, acc, lo, (q / p.tiles_y) * BX, (q % p.tiles_y) * BY, m_org, wn);
+    store_gw_tile<FM, FN>(p, stager, acc, lo, (q / p.tiles_y) * BX, (q % p.tiles_y) * BY, wt);
   }
 }
 
@@ -396,23 +471,54 @@ extern "C" int64_t momoe_wgrad_workspace_bytes(int64_t N, int64_t X, int64_t Y, 
          MOMOE_WGRAD_PARTIAL_BYTES;
 }
 
-extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gather,
-                           const void* B_rows, int64_t ldb, const int32_t* b_gather,
+namespace {
+template <class AOp, class BOp, int FM, int FN>
+int launch_wgrad(const WgradArgs& a, bool can_cut, int grid, hipStream_t st) {
+  static std::once_flag once, once_cut, once_reduce;
+  if (!can_cut) {
+    allow_lds(wgrad_kernel<false, AOp, BOp, FM, FN>, kWgradLds, once);
+    wgrad_kernel<false, AOp, BOp, FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
+  } else {
+    allow_lds(wgrad_kernel<true, AOp, BOp, FM, FN>, kWgradLds, once_cut);
+    allow_lds(wgrad_reduce_kernel<FM, FN>, kWgradLds, once_reduce);
+    wgrad_kernel<true, AOp, BOp, FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
+    wgrad_reduce_kernel<FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
+  }
+  return launch_status();
+}
+}  // namespace
+
+extern "C" int64_t momoe_padded_rows(int64_t Msum, int64_t N) {
+  if (Msum < 0 || N < 0) return -1;
+  return ((Msum + 31) & ~(int64_t)31) + 32 * N;
+}
+
+extern "C" int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32_t* a_gather,
+                           const void* B, int64_t ldb, int b_layout, const int32_t* b_gather,
                            const int32_t* cumsums_N1, void* GW_NXY, int64_t M, int64_t N,
                            int64_t X, int64_t Y, int64_t Msum, void* workspace,
                            int64_t workspace_bytes, void* stream) {
-  if (!A_rows || !B_rows || !cumsums_N1 || !GW_NXY) return MOMOE_ERR_BAD_ARG;
-  if (M <= 0 || N <= 0 || X <= 0 || Y <= 0 || Msum <= 0 || lda < X || ldb < Y)
+  if (!A || !B || !cumsums_N1 || !GW_NXY) return MOMOE_ERR_BAD_ARG;
+  if (M <= 0 || N <= 0 || X <= 0 || Y <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
+  const bool at = a_layout == MOMOE_LAYOUT_TRANSPOSED, bt = b_layout == MOMOE_LAYOUT_TRANSPOSED;
+  if ((!at && a_layout != MOMOE_LAYOUT_ROWS) || (!bt && b_layout != MOMOE_LAYOUT_ROWS))
+    return MOMOE_ERR_BAD_ARG;
+  if (at && bt) return MOMOE_ERR_UNSUPPORTED;  // one operand at most is handed over transposed
+  const int64_t mpad = momoe_padded_rows(Msum, N);
+  if (lda < X || ldb < Y || (at && a_gather != nullptr) || (bt && b_gather != nullptr))
     return MOMOE_ERR_BAD_ARG;
   if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace) || ((uintptr_t)workspace & 15))
     return MOMOE_ERR_BAD_ARG;
   if (X % 8 != 0 || Y % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return MOMOE_ERR_UNSUPPORTED;
-  if (((uintptr_t)A_rows & 15) || ((uintptr_t)B_rows & 15) || ((uintptr_t)GW_NXY & 7))
+  if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)GW_NXY & 7))
     return MOMOE_ERR_BAD_ARG;
-  if (Msum >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20)) return MOMOE_ERR_UNSUPPORTED;
+  if (Msum >= (1ll << 31) || mpad >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20))
+    return MOMOE_ERR_UNSUPPORTED;
   // rows are addressed with 32-bit byte offsets from the matrix base (gathered: M rows) or from
-  // the first row of an expert's piece (an expert holds a token at most once: at most M rows)
-  if (M * lda * 2 >= (1ll << 32) || M * ldb * 2 >= (1ll << 32)) return MOMOE_ERR_UNSUPPORTED;
+  // the first row of an expert's piece (an expert holds a token at most once: at most M rows);
+  // a transposed operand needs no such offsets (a stage is one contiguous block)
+  if ((!at && M * lda * 2 >= (1ll << 32)) || (!bt && M * ldb * 2 >= (1ll << 32)))
+    return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
   // the per-expert prefix sums live in LDS while the work is dealt out; work items are
   // counted in 32 bits (every expert has its tiles, the cut ones at most ws_tiles more)
@@ -429,20 +535,13 @@ extern "C" int momoe_wgrad(const void* A_rows, int64_t lda, const int32_t* a_gat
     const int64_t stages = (int64_t)tiles_x * tiles_y * (Msum / kBK + N);
     kc = (int)std::min<int64_t>(0x7fffffff, std::max<int64_t>(kMinChunk, cdiv64(stages, ws_tiles)));
   }
-  WgradArgs a{(const bf16*)A_rows, lda, a_gather, (const bf16*)B_rows, ldb, b_gather, cumsums_N1,
+  WgradArgs a{(const bf16*)A, lda, a_gather, (const bf16*)B, ldb, b_gather, cumsums_N1,
               (bf16*)GW_NXY, (float*)workspace, kc, (int)N, (int)X, (int)Y, tiles_x, tiles_y,
-              (int)Msum};
+              (int)Msum, clock_trace_buffer()};
   // an expert holds at most M rows: if that is short of the cutting length, nothing is cut
   const bool can_cut = kc != 0x7fffffff && cdiv64(std::min(M, Msum), kBK) >= 2 * (int64_t)kc;
-  static std::once_flag once, once_cut, once_reduce;
-  if (!can_cut) {
-    allow_lds(wgrad_kernel<false>, kWgradLds, once);
-    wgrad_kernel<false><<<grid, kThreads, kWgradLds, (hipStream_t)stream>>>(a);
-  } else {
-    allow_lds(wgrad_kernel<true>, kWgradLds, once_cut);
-    allow_lds(wgrad_reduce_kernel, kWgradLds, once_reduce);
-    wgrad_kernel<true><<<grid, kThreads, kWgradLds, (hipStream_t)stream>>>(a);
-    wgrad_reduce_kernel<<<grid, kThreads, kWgradLds, (hipStream_t)stream>>>(a);
-  }
-  return launch_status();
+  hipStream_t st = (hipStream_t)stream;
+  if (at) return launch_wgrad<TransposedOperand, RowsOperand, 4, 2>(a, can_cut, grid, st);
+  if (bt) return launch_wgrad<RowsOperand, TransposedOperand, 2, 4>(a, can_cut, grid, st);
+  return launch_wgrad<RowsOperand, RowsOperand, 4, 2>(a, can_cut, grid, st);
 }

@@ -30,6 +30,7 @@ _int = ctypes.c_int
 _SIGNATURES = {
     "momoe_abi_version": (_int, []),
     "momoe_status_string": (ctypes.c_char_p, [_int]),
+    "momoe_set_clock_trace": (_int, [_p]),
     "momoe_tile_table_ints": (_i64, [_i64, _i64, _i64, _int]),
     "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
     "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
@@ -42,15 +43,16 @@ _SIGNATURES = {
                                     _i64, _p]),
     "momoe_combine": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "momoe_dgrad_h": (_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
-    "momoe_lin1_swiglu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _p,
+    "momoe_lin1_swiglu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _i64, _p,
                                      _i64, _i64, _i64, _i64, _i64, _p]),
-    "momoe_swiglu_bwd_saved": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _i64, _p, _p, _p, _i64,
+    "momoe_swiglu_bwd_saved": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _i64, _p, _p, _i64, _p, _i64,
                                       _i64, _i64, _i64, _i64, _p]),
     "momoe_gs_scatter": (_int, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _p]),
     "momoe_dgrad_x": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "momoe_wgrad_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
-    "momoe_wgrad": (_int, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p,
-                           _i64, _p]),
+    "momoe_padded_rows": (_i64, [_i64, _i64]),
+    "momoe_wgrad": (_int, [_p, _i64, _int, _p, _p, _i64, _int, _p, _p, _p, _i64, _i64, _i64, _i64,
+                           _i64, _p, _i64, _p]),
     "momoe_router_fwd": (_int, [_p, _int, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p]),
     "momoe_router_bwd": (_int, [_p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p]),
 }
@@ -88,6 +90,25 @@ class kernel_timer:
     def durations_ms(self):
         torch.cuda.synchronize()
         return [(name, a.elapsed_time(b)) for name, a, b in self.records]
+
+
+class clock_trace:
+    """Context manager: average shader clock (MHz) under the grouped-GEMM kernels launched
+    inside it, from the in-kernel clock64() / wall_clock64() counters (momoe_set_clock_trace)."""
+
+    def __enter__(self):
+        self.ticks = torch.zeros(2, dtype=torch.int64, device="cuda")
+        _lib.momoe_set_clock_trace(self.ticks.data_ptr())
+        return self
+
+    def __exit__(self, *exc):
+        _lib.momoe_set_clock_trace(None)
+        return False
+
+    def mhz(self):
+        torch.cuda.synchronize()
+        c, w = self.ticks.tolist()
+        return 100.0 * c / w if w else float("nan")
 
 
 def _call(name, *args):
@@ -188,24 +209,22 @@ def dgrad_h(Gy_MD, Wl2_NHD, idx, table, u):
                               idx.numel(), _stream())
 
 
-def lin1_swiglu_bwd(x_MD, Wl1_ND2H, idx, table, u, s_NM, row_lo, gz, hs, gs_part):
+def lin1_swiglu_bwd(x_MD, Wl1_ND2H, idx, table, u, s_NM, row_lo, gz, hsT, gs_part):
     _need_cuda(x_MD, Wl1_ND2H, u, s_NM)
     M, D = x_MD.shape
     N, _, H2 = Wl1_ND2H.shape
     _call("momoe_lin1_swiglu_bwd", _ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(u),
-                                      _ptr(s_NM), s_NM.stride(0), s_NM.stride(1), row_lo, _ptr(gz),
-                                      _ptr(hs), _ptr(gs_part), M, D, H2 // 2, N, idx.numel(),
-                                      _stream())
+          _ptr(s_NM), s_NM.stride(0), s_NM.stride(1), row_lo, _ptr(gz), _ptr(hsT), hsT.shape[1],
+          _ptr(gs_part), M, D, H2 // 2, N, idx.numel(), _stream())
 
 
-def swiglu_bwd_saved(ab_save, u, s_NM, idx, cumsums, Msave, gz, hs, gs_part):
+def swiglu_bwd_saved(ab_save, u, s_NM, idx, cumsums, Msave, gz, hsT, gs_part):
     _need_cuda(ab_save, u, s_NM)
     N, M = s_NM.shape
     H = u.shape[1]
     _call("momoe_swiglu_bwd_saved", _ptr(ab_save), _ptr(u), _ptr(s_NM), s_NM.stride(0),
-                                       s_NM.stride(1), _ptr(idx), _ptr(cumsums), Msave, _ptr(gz),
-                                       _ptr(hs), _ptr(gs_part), gs_part.shape[0], M, H, N,
-                                       idx.numel(), _stream())
+          s_NM.stride(1), _ptr(idx), _ptr(cumsums), Msave, _ptr(gz), _ptr(hsT), hsT.shape[1],
+          _ptr(gs_part), gs_part.shape[0], M, H, N, idx.numel(), _stream())
 
 
 def gs_scatter(gs_part, idx, cumsums, Gs_NM):
@@ -224,16 +243,26 @@ def wgrad_workspace_bytes(N, X, Y, Msum):
     return _lib.momoe_wgrad_workspace_bytes(N, X, Y, Msum)
 
 
-def wgrad(A_rows, a_gather, B_rows, b_gather, cumsums, GW_NXY, M, Msum, workspace_bytes=None):
-    """workspace_bytes: scratch for the partial tiles of experts with many rows; default = the
+def padded_rows(Msum, N):
+    return _lib.momoe_padded_rows(Msum, N)
+
+
+def wgrad(A, a_gather, B, b_gather, cumsums, GW_NXY, M, Msum, workspace_bytes=None,
+          a_transposed=False, b_transposed=False):
+    """GW[i] = A_i^T . B_i over the sorted rows of expert i.  An operand is [row, feature]
+    (optionally gathered) or, with *_transposed, [padded sorted row / 32, feature, 32] as written
+    by the SwiGLU backward kernels.
+    workspace_bytes: scratch for the partial tiles of experts with many rows; default = the
     most the library can use for this shape, 0 = never cut an expert."""
     N, X, Y = GW_NXY.shape
     if workspace_bytes is None:
         workspace_bytes = wgrad_workspace_bytes(N, X, Y, Msum)
     ws = torch.empty(workspace_bytes, device=GW_NXY.device, dtype=torch.uint8) if workspace_bytes else None
-    _call("momoe_wgrad", _ptr(A_rows), A_rows.stride(0), _ptr(a_gather), _ptr(B_rows),
-                            B_rows.stride(0), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X,
-                            Y, Msum, _ptr(ws), workspace_bytes, _stream())
+    lda = A.shape[1] if a_transposed else A.stride(0)
+    ldb = B.shape[1] if b_transposed else B.stride(0)
+    _call("momoe_wgrad", _ptr(A), lda, int(a_transposed), _ptr(a_gather), _ptr(B),
+          ldb, int(b_transposed), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X, Y,
+          Msum, _ptr(ws), workspace_bytes, _stream())
 
 
 # ---------------------------------------------------------------- router

@@ -118,13 +118,15 @@ class MoEFunction(torch.autograd.Function):
             # SwiGLU backward: rows with saved a|b read them; the others recompute a|b = x.Wl1
             # and consume them straight from the GEMM's accumulators
             gz = torch.empty((msum, 2 * H), device=dev, dtype=torch.bfloat16)
-            hs = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
+            # s*h in groups of 32 padded sorted rows, feature-major inside a group: the layout
+            # the Wl2 gradient reads fastest
+            hsT = torch.empty((_hip.padded_rows(msum, N) // 32, H, 32), device=dev, dtype=torch.bfloat16)
             nparts = (H + _hip.GS_BLOCK - 1) // _hip.GS_BLOCK
             gs_part = torch.empty((nparts, msum), device=dev, dtype=torch.float32)
             if msave > 0:
-                _hip.swiglu_bwd_saved(ab_save, u, s, idx, cumsums, msave, gz, hs, gs_part)
+                _hip.swiglu_bwd_saved(ab_save, u, s, idx, cumsums, msave, gz, hsT, gs_part)
             if msave < msum:
-                _hip.lin1_swiglu_bwd(x_MD, W1, idx, table, u, s, msave, gz, hs, gs_part)
+                _hip.lin1_swiglu_bwd(x_MD, W1, idx, table, u, s, msave, gz, hsT, gs_part)
             del u
 
             G_s = None
@@ -135,13 +137,13 @@ class MoEFunction(torch.autograd.Function):
 
             # scratch for the weight gradients of experts with many rows: what the library can
             # use, but no more than u occupied (just freed, so the peak does not move)
-            ws_cap = hs.numel() * hs.element_size()
+            ws_cap = msum * H * 2
             G_W2 = None
             if need_w2:
                 G_W2 = torch.empty_like(W2)
-                _hip.wgrad(hs, None, Gy, idx, cumsums, G_W2, M, msum,
+                _hip.wgrad(hsT, None, Gy, idx, cumsums, G_W2, M, msum, a_transposed=True,
                            workspace_bytes=min(ws_cap, _hip.wgrad_workspace_bytes(N, H, D, msum)))
-            del hs
+            del hsT
 
             G_W1 = None
             if need_w1:
