@@ -106,6 +106,45 @@ def test_weight_gradient_of_cut_experts(gather_a):
     assert torch.equal(out[need][1:3], out[0][1:3])  # uncut experts: bit-identical
 
 
+@pytest.mark.parametrize("sizes,M", [([300, 0, 17, 1000, 64], 1000), ([20000, 3, 0, 5000], 20000)])
+def test_weight_gradient_from_a_transposed_operand(sizes, M):
+    # either operand handed over as [padded sorted row / 32, feature, 32] (the layout the SwiGLU
+    # backward writes s*h in): same result as from the row layout, against a plain fp32 matmul
+    from momoe_amd import _hip
+    dev = "cuda:0"
+    N, X, Y = len(sizes), 320, 512
+    msum = sum(sizes)
+    g = torch.Generator(device=dev).manual_seed(5)
+    c = [0] + list(torch.tensor(sizes).cumsum(0).tolist())
+    cumsums = torch.tensor(c, dtype=torch.int32, device=dev)
+    A = torch.randn(msum, X, generator=g, device=dev).to(torch.bfloat16)
+    B = torch.randn(msum, Y, generator=g, device=dev).to(torch.bfloat16)
+
+    def grouped(rows):
+        F = rows.shape[1]
+        mpad = _hip.padded_rows(msum, N)
+        assert mpad == (msum + 31) // 32 * 32 + 32 * N
+        # garbage outside the experts' own 32-row groups must not matter; zeros inside them do
+        T = torch.full((F, mpad), float("nan"), device=dev, dtype=rows.dtype)
+        for e in range(N):
+            p0 = (c[e] + 31) // 32 * 32 + 32 * e
+            n = c[e + 1] - c[e]
+            T[:, p0:p0 + (n + 31) // 32 * 32] = 0
+            T[:, p0:p0 + n] = rows[c[e]:c[e + 1]].T
+        return T.reshape(F, mpad // 32, 32).permute(1, 0, 2).contiguous()
+
+    want = torch.stack([A[c[e]:c[e + 1]].float().T @ B[c[e]:c[e + 1]].float() for e in range(N)])
+    for kw, a, b in ((dict(a_transposed=True), grouped(A), B), (dict(b_transposed=True), A, grouped(B))):
+        for ws in (None, 0):
+            GW = torch.full((N, X, Y), float("nan"), device=dev, dtype=torch.bfloat16)
+            _hip.wgrad(a, None, b, None, cumsums, GW, M, msum, workspace_bytes=ws, **kw)
+            torch.cuda.synchronize()
+            for e in range(N):
+                assert_close(GW[e], want[e], f"GW[{e}] {kw} ws={ws}", rel=5e-3)
+    with pytest.raises(RuntimeError):  # both transposed: refused
+        _hip.wgrad(grouped(A), None, grouped(B), None, cumsums, GW, M, msum, a_transposed=True, b_transposed=True)
+
+
 def test_experts_without_tokens_get_zero_weight_grads():
     M, D, H, N, K = 256, 128, 64, 8, 2
     x, W1, W2, _, _, dy = make_layer_inputs(M, D, H, N, K, seed=9)
