@@ -315,6 +315,9 @@ __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
 }
 
 // out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.
+// The row numbers and then the rows are fetched 8 at a time with unconditional loads (a missing
+// pair, inv = -1, is pointed at row 0 and left out of the sum): loads under a branch would be
+// waited for one by one.
 __global__ __launch_bounds__(256) void combine_kernel(const bf16* __restrict__ rows,
                                                       const int32_t* __restrict__ inv,
                                                       bf16* __restrict__ out, int D, int K,
@@ -322,12 +325,21 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16* __restrict__ r
   const int64_t m = blockIdx.x;
   for (int c = threadIdx.x; c < D / 8; c += blockDim.x) {
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k = 0; k < K; ++k) {
-      const int32_t r = inv[m * K + k];
-      if ((uint32_t)r >= (uint64_t)msum) continue;
-      const bf16x8 v = *(const bf16x8*)(rows + (int64_t)r * D + c * 8);
+    for (int k0 = 0; k0 < K; k0 += 8) {
+      int32_t r[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)v[e];
+      for (int j = 0; j < 8; ++j) r[j] = inv[m * K + min(k0 + j, K - 1)];
+      bf16x8 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool ok = k0 + j < K && (uint32_t)r[j] < (uint64_t)msum;
+        v[j] = *(const bf16x8*)(rows + (int64_t)(ok ? r[j] : 0) * D + c * 8);
+        r[j] = ok ? 1 : 0;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += r[j] ? (float)v[j][e] : 0.0f;
     }
     bf16x8 o;
 #pragma unroll
