@@ -102,22 +102,25 @@ int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n, int64_t s
 /* ---- experts forward -----------------------------------------------------
  * momoe_lin1_swiglu_fwd replaces lin1_kernel (momoe/momoe.py:69-152):
  *   [a|b] = x[idx[r]] @ Wl1[i]  (fp32 accumulate), h[r] = bf16(a * b * sigmoid(b)).
- * x_MD bf16 [M,D]; Wl1_ND2H bf16 [N,D,2H]; h_MsumH bf16 [Msum,H] (may be NULL:
- * then only a|b is produced and row tiles entirely below ab_row_lo are skipped);
+ * x_MD bf16 [M,D]; Wl1_ND2H bf16 [N,D,2H]; h_blocked bf16 [H/32][Msum][32]: h[r][j] at
+ * [((j / 32) * Msum + r) * 32 + j % 32], the layout momoe_lin2_scale_fwd reads (its contraction
+ * runs over j: 32 of them for consecutive rows are one contiguous block).  h_blocked may be NULL:
+ * then only a|b is produced and row tiles entirely below ab_row_lo are skipped;
  * ab_rows bf16 [*,2H] indexed by the sorted row r (may be NULL): rows with
  * ab_row_lo <= r < ab_row_hi receive bf16(a)|bf16(b) (the selective save of
  * :141-145 with lo=0, hi=Msave).
  */
 int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
-                          const int32_t* tile_table, void* h_MsumH,
+                          const int32_t* tile_table, void* h_blocked,
                           void* ab_rows, int64_t ab_row_lo, int64_t ab_row_hi,
                           int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
 
 /* momoe_lin2_scale_fwd replaces lin2_kernel (momoe/momoe.py:161-237):
  *   ys[r] = bf16( (h[r] @ Wl2[i]) * s[i, idx[r]] ), rows kept in sorted order.
+ * h_blocked as written by momoe_lin1_swiglu_fwd.
  * s_NM fp32, element (i,m) at s[i*s_stride_n + m*s_stride_m]. ys_MsumD bf16 [Msum,D].
  */
-int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD,
+int momoe_lin2_scale_fwd(const void* h_blocked, const void* Wl2_NHD,
                          const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
                          const int32_t* idx_Msum, const int32_t* tile_table, void* ys_MsumD,
                          int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
@@ -140,11 +143,14 @@ int momoe_combine(const void* rows_MsumD, const int32_t* inv_MK, void* out_MD,
  * momoe_lin1_swiglu_bwd, for the sorted rows without saved a|b:
  *   a|b  = x[idx[r]] @ Wl1[i]   (fp32, kept in registers)
  *   s    = s_NM[i, idx[r]],  sig = sigmoid(b)
- *   gz[r] = bf16( s u b sig | s u a sig (1 + b (1 - sig)) )       [G_a | G_b]
+ *   gz[r] = bf16( s u b sig | s u a sig (1 + b (1 - sig)) )       [G_a | G_b], 2H columns
  *   hs    = bf16( s a b sig )       (h pre-scaled by the gate weight, for the Wl2 gradient)
  *   gs_part[p][r] = sum over the p-th block of MOMOE_GS_BLOCK hidden columns of u a b sig
  * (sum_p gs_part[p][r] = G_y[idx[r]] . (h[r] @ Wl2[i]) = dL/ds, by associativity).
  * gs_part fp32 [ceil(H/MOMOE_GS_BLOCK)][Msum].
+ * gz is written k-blocked, gz_blocked bf16 [2H/32][Msum][32]: gz[r][j] at
+ * [((j / 32) * Msum + r) * 32 + j % 32] -- the layout momoe_dgrad_x contracts over and
+ * MOMOE_LAYOUT_KBLOCKED of momoe_wgrad.
  * hs is written in the layout MOMOE_LAYOUT_TRANSPOSED of momoe_wgrad, zero padding included:
  * hsT_GH32 bf16 [momoe_padded_rows(Msum, N) / 32][ld_hsT][32], ld_hsT >= H a multiple of 8.
  *
@@ -166,14 +172,14 @@ int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32_t* idx_Msu
 int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H, const int32_t* idx_Msum,
                           const int32_t* tile_table, const void* u_MsumH,
                           const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
-                          int64_t row_lo, void* gz_Msum2H, void* hsT_GH32, int64_t ld_hsT,
+                          int64_t row_lo, void* gz_blocked, void* hsT_GH32, int64_t ld_hsT,
                           float* gs_part,
                           int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
 
 int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH,
                            const float* s_NM, int64_t s_stride_n, int64_t s_stride_m,
                            const int32_t* idx_Msum, const int32_t* cumsums_N1, int64_t Msave,
-                           void* gz_Msum2H, void* hsT_GH32, int64_t ld_hsT,
+                           void* gz_blocked, void* hsT_GH32, int64_t ld_hsT,
                            float* gs_part, int64_t nparts,
                            int64_t M, int64_t H, int64_t N, int64_t Msum, void* stream);
 
@@ -187,9 +193,9 @@ int momoe_gs_scatter(const float* gs_part, int64_t nparts, const int32_t* idx_Ms
 
 /* momoe_dgrad_x replaces the GEMM of lin1_backward_kernel (momoe/momoe.py:662-681):
  *   gxs[r] = bf16( gz[r] @ Wl1[i]^T ), rows kept in sorted order; follow with
- *   momoe_combine to obtain G_x.
+ *   momoe_combine to obtain G_x.  gz_blocked as written by the SwiGLU backward entry points.
  */
-int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* tile_table,
+int momoe_dgrad_x(const void* gz_blocked, const void* Wl1_ND2H, const int32_t* tile_table,
                   void* gxs_MsumD, int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum,
                   void* stream);
 
@@ -209,10 +215,13 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
  *                            one, which the kernel reads from LDS at twice the rate of the row
  *                            layout, and each 32-row stage of a tile is one contiguous block.
  *                            At most one operand may be transposed.
+ *   MOMOE_LAYOUT_KBLOCKED    (B only) bf16 [features/32][ld][32] with ld >= Msum = rows of the
+ *                            matrix, no gather: B(r, y) = B[((y / 32) * ld + r) * 32 + y % 32];
+ *                            Y a multiple of 32.  This is how gz is written.
  * M = number of tokens (rows of a gathered matrix, and the most rows an expert can hold);
  * M * ld * 2 bytes (row layout) must stay below 4 GiB.  Experts without rows get exact zeros.
  * Wl2 gradient: A = hs (transposed, X=H), B = G_y gathered by idx (Y=D).
- * Wl1 gradient: A = x gathered by idx (X=D), B = gz (rows, Y=2H).
+ * Wl1 gradient: A = x gathered by idx (X=D), B = gz (k-blocked, Y=2H).
  * workspace: device scratch (16-byte aligned, contents undefined on entry and exit) for
  * fp32 partial tiles of MOMOE_WGRAD_PARTIAL_BYTES each.  An expert that holds many times
  * the average number of rows is contracted in several pieces so that its tiles do not
@@ -225,6 +234,7 @@ int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H, const int32_t* ti
 #define MOMOE_WGRAD_PARTIAL_BYTES 262144
 #define MOMOE_LAYOUT_ROWS 0
 #define MOMOE_LAYOUT_TRANSPOSED 1
+#define MOMOE_LAYOUT_KBLOCKED 2
 int64_t momoe_padded_rows(int64_t Msum, int64_t N);
 int64_t momoe_wgrad_workspace_bytes(int64_t N, int64_t X, int64_t Y, int64_t Msum);
 int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32_t* a_gather,

@@ -12,6 +12,7 @@ constexpr int BN = 256;
 constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 rows x 64 columns
 using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
 using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
+using BlockedA = RBlockedDma<BM>;  // sorted rows of a k-blocked intermediate (gz)
 using Ring = StageRing<RowsA, RowsB>;
 constexpr size_t kBwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
 
@@ -153,9 +154,9 @@ __global__ __launch_bounds__(256) void swiglu_bwd_saved_kernel(SavedArgs p) {
         gb[e] = (bf16)(gh * a * sg * (1.0f + b * (1.0f - sg)));
         hv[e] = (bf16)(rowok ? sv * hval : 0.0f);
       }
-      if (rowok) {
-        *(bf16x8*)(p.gz + r * 2 * H + c) = ga;
-        *(bf16x8*)(p.gz + r * 2 * H + H + c) = gb;
+      if (rowok) {  // gz is k-blocked: [2H/32][Msum][32]
+        *(bf16x8*)(p.gz + ((int64_t)(c >> 5) * p.msum + r) * 32 + (c & 31)) = ga;
+        *(bf16x8*)(p.gz + ((int64_t)((H + c) >> 5) * p.msum + r) * 32 + (c & 31)) = gb;
       }
     }
     // transposed staging: column-major, the four 8-row groups of a column rotated by the
@@ -188,6 +189,7 @@ struct DxArgs {
   const int32_t* table;
   bf16* gxs;
   int D, H;
+  int64_t msum;
   unsigned long long* clk;
 };
 
@@ -200,11 +202,11 @@ struct DxProg {
 
   __device__ __forceinline__ void gather(const TileCoord&, Prep&) const {}
   __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
-  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, RowsA& A, RowsB& B) const {
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, BlockedA& A, RowsB& B) const {
     const int D = p.D, H2 = 2 * p.H;
     const bf16* w = p.w1 + (int64_t)t.expert * D * H2;
     const int d0 = t.tn * BN;
-    A.init(p.gz + (int64_t)t.row0 * H2, [&](int r, int) { return (uint32_t)(min(r, t.rows - 1) * 2 * H2); });
+    A.init(p.gz, p.msum, t.row0, t.rows);
     B.init(w, [&](int r, int) { return (uint32_t)min(d0 + r, D - 1) * (uint32_t)(2 * H2); });
   }
   __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
@@ -230,7 +232,7 @@ struct DxProg {
 
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
   const ClockTrace trace(p.clk);
-  Ring ring(dyn_lds());
+  StageRing<BlockedA, RowsB> ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
@@ -291,15 +293,15 @@ extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32
 extern "C" int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH, const float* s_NM,
                                       int64_t s_stride_n, int64_t s_stride_m,
                                       const int32_t* idx_Msum, const int32_t* cumsums_N1,
-                                      int64_t Msave, void* gz_Msum2H, void* hsT_GH32,
+                                      int64_t Msave, void* gz_blocked, void* hsT_GH32,
                                       int64_t ld_hsT, float* gs_part, int64_t nparts, int64_t M,
                                       int64_t H, int64_t N, int64_t Msum, void* stream) {
-  if (!ab_save || !u_MsumH || !s_NM || !idx_Msum || !cumsums_N1 || !gz_Msum2H || !hsT_GH32 ||
+  if (!ab_save || !u_MsumH || !s_NM || !idx_Msum || !cumsums_N1 || !gz_blocked || !hsT_GH32 ||
       !gs_part)
     return MOMOE_ERR_BAD_ARG;
   if (Msave < 0 || Msave > Msum || nparts <= 0 || M <= 0 || H <= 0 || N <= 0 || Msum <= 0)
     return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_Msum2H) || !aligned16(hsT_GH32))
+  if (!aligned16(ab_save) || !aligned16(u_MsumH) || !aligned16(gz_blocked) || !aligned16(hsT_GH32))
     return MOMOE_ERR_BAD_ARG;
   const int64_t mpad = momoe_padded_rows(Msum, N);
   if (ld_hsT < H || ld_hsT % 8 != 0) return MOMOE_ERR_BAD_ARG;
@@ -307,7 +309,7 @@ extern "C" int momoe_swiglu_bwd_saved(const void* ab_save, const void* u_MsumH, 
     return MOMOE_ERR_UNSUPPORTED;
   if (Msave == 0) return MOMOE_OK;
   SavedArgs a{(const bf16*)ab_save, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m, idx_Msum,
-              cumsums_N1, (bf16*)gz_Msum2H, (bf16*)hsT_GH32, ld_hsT, gs_part, (int)nparts, Msum,
+              cumsums_N1, (bf16*)gz_blocked, (bf16*)hsT_GH32, ld_hsT, gs_part, (int)nparts, Msum,
               Msave, (int)H, (int)N, (int)M};
   const int64_t spans = cdiv64(H, kSavedSpan);
   if (spans > nparts || spans > 65535) return MOMOE_ERR_BAD_ARG;  // nparts = ceil(H / MOMOE_GS_BLOCK)
@@ -326,16 +328,16 @@ extern "C" int momoe_gs_scatter(const float* gs_part, int64_t nparts, const int3
   return launch_status();
 }
 
-extern "C" int momoe_dgrad_x(const void* gz_Msum2H, const void* Wl1_ND2H,
+extern "C" int momoe_dgrad_x(const void* gz_blocked, const void* Wl1_ND2H,
                              const int32_t* tile_table, void* gxs_MsumD, int64_t M, int64_t D,
                              int64_t H, int64_t N, int64_t Msum, void* stream) {
-  if (!gz_Msum2H || !Wl1_ND2H || !tile_table || !gxs_MsumD) return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(gz_Msum2H) || !aligned16(Wl1_ND2H) || ((uintptr_t)gxs_MsumD & 7))
+  if (!gz_blocked || !Wl1_ND2H || !tile_table || !gxs_MsumD) return MOMOE_ERR_BAD_ARG;
+  if (!aligned16(gz_blocked) || !aligned16(Wl1_ND2H) || ((uintptr_t)gxs_MsumD & 7))
     return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
-  DxArgs a{(const bf16*)gz_Msum2H, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
-           (int)H, clock_trace_buffer()};
+  DxArgs a{(const bf16*)gz_blocked, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
+           (int)H, Msum, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(dgrad_x_kernel, kBwdLds, once);
   dgrad_x_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);

@@ -9,6 +9,7 @@ constexpr int BM = MOMOE_TILE_ROWS;  // 256 sorted rows per tile
 constexpr int BN = 256;              // GEMM columns per tile
 constexpr int FM = 4, FN = 2;        // 2x4 waves, each 128 rows x 64 columns
 using RowsOp = RDma<BM>;             // token rows, k-contiguous
+using HRowsOp = RBlockedDma<BM>;     // rows of h, k-blocked
 using WeightOp = TDma;               // expert weights [k][col], k-strided
 using Ring = StageRing<RowsOp, WeightOp>;
 constexpr size_t kFwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
@@ -110,7 +111,14 @@ struct Lin1Prog {
                                        a[q][1] * b[q][1] * sigmoidf_fast(b[q][1]),
                                        a[q][2] * b[q][2] * sigmoidf_fast(b[q][2]),
                                        a[q][3] * b[q][3] * sigmoidf_fast(b[q][3])));
-        stager.flush(dst(p.h, H, 0, false));
+        // h is k-blocked for the next GEMM: this wave's 32 hidden columns are one k-block, so
+        // the fragment's rows are consecutive 64-byte pieces of memory
+        bf16* hblock = p.h + (int64_t)(j0 >> 5) * p.msum * 32;
+        stager.flush([&](int row, int col) -> bf16* {
+          const int rl = (tc.mbase + 32 * i) + row;
+          if (rl >= tc.rows || j0 >= H) return nullptr;
+          return hblock + ((int64_t)tc.row0 + rl) * 32 + col;
+        });
       }
       if (p.ab) {
 #pragma unroll
@@ -171,15 +179,19 @@ struct Lin1Prog {
       }
       const int rl0 = tc.mbase + 32 * i;  // first tile row of this fragment row
       const bool mine = rl0 >= rl_lo;      // wave-uniform
-      auto dst = [&](bf16* mat, int64_t ld, int col0) {
+      // gz is k-blocked ([2H/32][Msum][32], the layout dL/dx contracts over): this wave's 32
+      // columns of G_a are block j0/32, those of G_b block (H + j0)/32, and a fragment's rows are
+      // consecutive 64-byte pieces of memory
+      auto dst = [&](int block) {
+        bf16* base = p.gz + (int64_t)block * p.msum * 32;
         return [=, *this](int row, int col) -> bf16* {
           const int rl = rl0 + row;
-          if (rl >= tc.rows || j0 + col >= H || !mine) return nullptr;
-          return mat + ((int64_t)tc.row0 + rl) * ld + col0 + j0 + col;
+          if (rl >= tc.rows || j0 >= H || !mine) return nullptr;
+          return base + ((int64_t)tc.row0 + rl) * 32 + col;
         };
       };
-      stager.flush(dst(p.gz, 2 * H, 0));
-      stager1.flush(dst(p.gz, 2 * H, H));
+      stager.flush(dst(j0 >> 5));
+      stager1.flush(dst((H + j0) >> 5));
       // hs^T: the 32 x 32 fragment goes through the staging area transposed ([column][row],
       // the four 8-row groups of a column permuted so that the two half-waves, which write
       // columns 4 apart, use different banks) and leaves it as 8 consecutive rows of one column
@@ -254,6 +266,7 @@ struct Lin2Args {
   const int32_t* table;
   bf16* ys;
   int D, H;
+  int64_t msum;
   unsigned long long* clk;
 };
 
@@ -274,11 +287,11 @@ struct Lin2Prog {
 #pragma unroll
     for (int i = 0; i < FM; ++i) g.sv[i] = p.s[(int64_t)t.expert * p.ssn + (int64_t)g.tok[i] * p.ssm];
   }
-  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, RowsOp& A, WeightOp& B) const {
+  __device__ __forceinline__ void setup(const TileCoord& t, const Prep&, HRowsOp& A, WeightOp& B) const {
     const int D = p.D, H = p.H;
     const bf16* w = p.w2 + (int64_t)t.expert * H * D;
     const int d0 = t.tn * BN;
-    A.init(p.h + (int64_t)t.row0 * H, [&](int r, int) { return (uint32_t)(min(r, t.rows - 1) * 2 * H); });
+    A.init(p.h, p.msum, t.row0, t.rows);
     B.init(w, [&](int c) { return min(d0 + c, D - 8); }, D);
   }
   __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
@@ -305,7 +318,7 @@ struct Lin2Prog {
 
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
   const ClockTrace trace(p.clk);
-  Ring ring(dyn_lds());
+  StageRing<HRowsOp, WeightOp> ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
@@ -366,17 +379,17 @@ using namespace momoe;
 
 extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
                                      const int32_t* idx_Msum, const int32_t* tile_table,
-                                     void* h_MsumH, void* ab_rows, int64_t ab_row_lo,
+                                     void* h_blocked, void* ab_rows, int64_t ab_row_lo,
                                      int64_t ab_row_hi, int64_t M, int64_t D, int64_t H,
                                      int64_t N, int64_t Msum, void* stream) {
-  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || (!h_MsumH && !ab_rows))
+  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || (!h_blocked && !ab_rows))
     return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_MsumH & 15) ||
+  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_blocked & 15) ||
       ((uintptr_t)ab_rows & 15))
     return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
-  Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_MsumH,
+  Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_blocked,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
              nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, Msum, clock_trace_buffer()};
   static std::once_flag once;
@@ -388,15 +401,15 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
 extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
                                      const int32_t* idx_Msum, const int32_t* tile_table,
                                      const void* u_MsumH, const float* s_NM, int64_t s_stride_n,
-                                     int64_t s_stride_m, int64_t row_lo, void* gz_Msum2H,
+                                     int64_t s_stride_m, int64_t row_lo, void* gz_blocked,
                                      void* hsT_GH32, int64_t ld_hsT, float* gs_part, int64_t M,
                                      int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream) {
-  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || !u_MsumH || !s_NM || !gz_Msum2H ||
+  if (!x_MD || !Wl1_ND2H || !idx_Msum || !tile_table || !u_MsumH || !s_NM || !gz_blocked ||
       !hsT_GH32 || !gs_part)
     return MOMOE_ERR_BAD_ARG;
   if (row_lo < 0 || row_lo > Msum) return MOMOE_ERR_BAD_ARG;
   if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)u_MsumH & 7) ||
-      !aligned16(gz_Msum2H) || !aligned16(hsT_GH32))
+      !aligned16(gz_blocked) || !aligned16(hsT_GH32))
     return MOMOE_ERR_BAD_ARG;
   if (ld_hsT < H || ld_hsT % 8 != 0) return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
@@ -404,26 +417,26 @@ extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
   if (row_lo == Msum) return MOMOE_OK;
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, nullptr, nullptr,
              row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
-             (bf16*)gz_Msum2H, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
+             (bf16*)gz_blocked, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(lin1_swiglu_kernel<true>, kFwdLds, once);
   lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
-extern "C" int momoe_lin2_scale_fwd(const void* h_MsumH, const void* Wl2_NHD, const float* s_NM,
+extern "C" int momoe_lin2_scale_fwd(const void* h_blocked, const void* Wl2_NHD, const float* s_NM,
                                     int64_t s_stride_n, int64_t s_stride_m,
                                     const int32_t* idx_Msum, const int32_t* tile_table,
                                     void* ys_MsumD, int64_t M, int64_t D, int64_t H, int64_t N,
                                     int64_t Msum, void* stream) {
-  if (!h_MsumH || !Wl2_NHD || !s_NM || !idx_Msum || !tile_table || !ys_MsumD)
+  if (!h_blocked || !Wl2_NHD || !s_NM || !idx_Msum || !tile_table || !ys_MsumD)
     return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(h_MsumH) || !aligned16(Wl2_NHD) || ((uintptr_t)ys_MsumD & 7))
+  if (!aligned16(h_blocked) || !aligned16(Wl2_NHD) || ((uintptr_t)ys_MsumD & 7))
     return MOMOE_ERR_BAD_ARG;
   const int st = check_dims(M, D, H, N, Msum);
   if (st != MOMOE_OK) return st;
-  Lin2Args a{(const bf16*)h_MsumH, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
-             idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, clock_trace_buffer()};
+  Lin2Args a{(const bf16*)h_blocked, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
+             idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, Msum, clock_trace_buffer()};
   static std::once_flag once;
   allow_lds(lin2_scale_kernel, kFwdLds, once);
   lin2_scale_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);

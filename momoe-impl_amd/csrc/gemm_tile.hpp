@@ -162,6 +162,34 @@ struct RDma {
   }
 };
 
+// The same LDS stage fed from a k-blocked matrix: element (row, k) at
+// mat[((k / 32) * nrows + row) * 32 + k % 32].  Intermediates that this library both writes and
+// reads (h between the two forward GEMMs) are stored like this: a stage of consecutive rows is
+// one contiguous block of memory, fetched in whole 128-byte lines, where the row-major layout
+// asks for half a line per row and stage.
+template <int ROWS>
+struct RBlockedDma {
+  using R = RDma<ROWS>;
+  static constexpr int NCH = R::NCH;
+  static constexpr int LDS_ELEMS = R::LDS_ELEMS;
+  R r;
+  int64_t kstride;  // elements between consecutive k-blocks = 32 * rows of the matrix
+  // rows [row0, row0 + ROWS) of the matrix; rows >= nvalid (tile-local) are clamped to the last
+  __device__ __forceinline__ void init(const bf16* mat, int64_t nrows, int64_t row0, int nvalid) {
+    kstride = nrows * kBK;
+    r.init(mat + row0 * kBK, [&](int row, int) { return (uint32_t)min(row, nvalid - 1) * (uint32_t)(kBK * 2); });
+  }
+  __device__ __forceinline__ void issue(int kt, uint32_t stage) {
+    const int w = threadIdx.x >> 6;
+    const bf16* b = r.base + (int64_t)kt * kstride;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) dma16(b, r.off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
+  }
+  template <int S>
+  __device__ __forceinline__ void issue_head(uint32_t stage) { issue(S, stage); }
+  static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int r0, int kk) { return R::frag(stage, r0, kk); }
+};
+
 // ---- k-strided operand, 256 columns -----------------------------------------------------
 // LDS stage: k-row k at elements [256k, 256k+256); 16-byte piece p of the row is stored
 // at position p ^ swz(k), swz(k) = 4*(k&3) + 16*((k>>3)&1): the 8 k-rows x 64 bytes that one

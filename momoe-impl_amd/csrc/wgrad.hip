@@ -36,6 +36,30 @@ struct RowsOperand : TGatherDma {
     set_rows(gather_, ld_, rb, re);
   }
 };
+// "k-blocked" operand: sorted rows (no gather) of a matrix stored in blocks of 32 features,
+// feature f of row r at mat[((f / 32) * ld + r) * 32 + f % 32], ld = rows of the matrix (gz, as
+// the SwiGLU backward writes it for dL/dx).  Rows are the contraction index, as in the row layout,
+// and go through the same transposing LDS reads; the 32 rows x 32 features of a block are 2 KiB
+// of consecutive memory.
+struct BlockedRowsOperand : TGatherDma {
+  int64_t nrows;
+  __device__ __forceinline__ void begin_piece(const int32_t*, int64_t ld_, int rb, int re, int) {
+    nrows = ld_;
+    set_rows(nullptr, 32, rb, re);  // row pitch: 32 elements
+  }
+  // features [col0, col0+256) (col0 a multiple of 256); features >= ncols are clamped to col0
+  __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
+    mat = mat_ + ((int64_t)(col0 >> 5) * nrows + row_begin) * 32;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      int krow, c;
+      L::lane_piece(j, krow, c);
+      const int cc = col0 + c < ncols ? c : 0;
+      colb[j] = (uint32_t)(((int64_t)(cc >> 5) * nrows * 32 + (cc & 31)) * 2);
+    }
+  }
+};
+
 // "transposed" operand: groups of 32 padded sorted rows, feature-major inside a group: feature f
 // of padded sorted row p at mat[(p / 32) * ld * 32 + f * 32 + p % 32], ld >= number of features.
 // The 256 features x 32 rows of one stage are 16 KiB of consecutive memory.
@@ -501,15 +525,20 @@ extern "C" int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32
   if (!A || !B || !cumsums_N1 || !GW_NXY) return MOMOE_ERR_BAD_ARG;
   if (M <= 0 || N <= 0 || X <= 0 || Y <= 0 || Msum <= 0) return MOMOE_ERR_BAD_ARG;
   const bool at = a_layout == MOMOE_LAYOUT_TRANSPOSED, bt = b_layout == MOMOE_LAYOUT_TRANSPOSED;
-  if ((!at && a_layout != MOMOE_LAYOUT_ROWS) || (!bt && b_layout != MOMOE_LAYOUT_ROWS))
+  const bool bk = b_layout == MOMOE_LAYOUT_KBLOCKED;
+  if ((!at && a_layout != MOMOE_LAYOUT_ROWS) || (!bt && !bk && b_layout != MOMOE_LAYOUT_ROWS))
     return MOMOE_ERR_BAD_ARG;
-  if (at && bt) return MOMOE_ERR_UNSUPPORTED;  // one operand at most is handed over transposed
+  if (at && (bt || bk)) return MOMOE_ERR_UNSUPPORTED;  // one operand at most in a special layout
+  // k-blocked B: ldb = rows of the matrix; features in whole blocks; 8 blocks of a tile are
+  // addressed with 32-bit byte offsets
+  if (bk && (b_gather != nullptr || ldb < Msum || Y % 32 != 0 || 8 * ldb * 64 >= (1ll << 32)))
+    return b_gather != nullptr || ldb < Msum ? MOMOE_ERR_BAD_ARG : MOMOE_ERR_UNSUPPORTED;
   const int64_t mpad = momoe_padded_rows(Msum, N);
-  if (lda < X || ldb < Y || (at && a_gather != nullptr) || (bt && b_gather != nullptr))
+  if (lda < X || (!bk && ldb < Y) || (at && a_gather != nullptr) || (bt && b_gather != nullptr))
     return MOMOE_ERR_BAD_ARG;
   if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace) || ((uintptr_t)workspace & 15))
     return MOMOE_ERR_BAD_ARG;
-  if (X % 8 != 0 || Y % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return MOMOE_ERR_UNSUPPORTED;
+  if (X % 8 != 0 || Y % 8 != 0 || lda % 8 != 0 || (!bk && ldb % 8 != 0)) return MOMOE_ERR_UNSUPPORTED;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)GW_NXY & 7))
     return MOMOE_ERR_BAD_ARG;
   if (Msum >= (1ll << 31) || mpad >= (1ll << 31) || X > (1 << 20) || Y > (1 << 20))
@@ -517,7 +546,7 @@ extern "C" int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32
   // rows are addressed with 32-bit byte offsets from the matrix base (gathered: M rows) or from
   // the first row of an expert's piece (an expert holds a token at most once: at most M rows);
   // a transposed operand needs no such offsets (a stage is one contiguous block)
-  if ((!at && M * lda * 2 >= (1ll << 32)) || (!bt && M * ldb * 2 >= (1ll << 32)))
+  if ((!at && M * lda * 2 >= (1ll << 32)) || (!bt && !bk && M * ldb * 2 >= (1ll << 32)))
     return MOMOE_ERR_UNSUPPORTED;
   const int tiles_x = (int)cdiv64(X, BX), tiles_y = (int)cdiv64(Y, BY);
   // the per-expert prefix sums live in LDS while the work is dealt out; work items are
@@ -543,5 +572,6 @@ extern "C" int momoe_wgrad(const void* A, int64_t lda, int a_layout, const int32
   hipStream_t st = (hipStream_t)stream;
   if (at) return launch_wgrad<TransposedOperand, RowsOperand, 4, 2>(a, can_cut, grid, st);
   if (bt) return launch_wgrad<RowsOperand, TransposedOperand, 2, 4>(a, can_cut, grid, st);
+  if (bk) return launch_wgrad<RowsOperand, BlockedRowsOperand, 4, 2>(a, can_cut, grid, st);
   return launch_wgrad<RowsOperand, RowsOperand, 4, 2>(a, can_cut, grid, st);
 }

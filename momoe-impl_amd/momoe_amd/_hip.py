@@ -234,9 +234,10 @@ def gs_scatter(gs_part, idx, cumsums, Gs_NM):
 
 
 def dgrad_x(gz, Wl1_ND2H, table, gxs, M):
+    """gz k-blocked: [2H/32, Msum, 32]."""
     N, D, H2 = Wl1_ND2H.shape
     _call("momoe_dgrad_x", _ptr(gz), _ptr(Wl1_ND2H), _ptr(table), _ptr(gxs), M, D, H2 // 2, N,
-                              gz.shape[0], _stream())
+                              gz.shape[1], _stream())
 
 
 def wgrad_workspace_bytes(N, X, Y, Msum):
@@ -248,10 +249,10 @@ def padded_rows(Msum, N):
 
 
 def wgrad(A, a_gather, B, b_gather, cumsums, GW_NXY, M, Msum, workspace_bytes=None,
-          a_transposed=False, b_transposed=False):
+          a_transposed=False, b_transposed=False, b_kblocked=False):
     """GW[i] = A_i^T . B_i over the sorted rows of expert i.  An operand is [row, feature]
     (optionally gathered) or, with *_transposed, [padded sorted row / 32, feature, 32] as written
-    by the SwiGLU backward kernels.
+    by the SwiGLU backward kernels; B may also be k-blocked, [feature / 32, row, 32] (gz).
     workspace_bytes: scratch for the partial tiles of experts with many rows; default = the
     most the library can use for this shape, 0 = never cut an expert."""
     N, X, Y = GW_NXY.shape
@@ -259,9 +260,9 @@ def wgrad(A, a_gather, B, b_gather, cumsums, GW_NXY, M, Msum, workspace_bytes=No
         workspace_bytes = wgrad_workspace_bytes(N, X, Y, Msum)
     ws = torch.empty(workspace_bytes, device=GW_NXY.device, dtype=torch.uint8) if workspace_bytes else None
     lda = A.shape[1] if a_transposed else A.stride(0)
-    ldb = B.shape[1] if b_transposed else B.stride(0)
+    ldb = B.shape[1] if (b_transposed or b_kblocked) else B.stride(0)
     _call("momoe_wgrad", _ptr(A), lda, int(a_transposed), _ptr(a_gather), _ptr(B),
-          ldb, int(b_transposed), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X, Y,
+          ldb, 2 if b_kblocked else int(b_transposed), _ptr(b_gather), _ptr(cumsums), _ptr(GW_NXY), M, N, X, Y,
           Msum, _ptr(ws), workspace_bytes, _stream())
 
 

@@ -72,7 +72,8 @@ class MoEFunction(torch.autograd.Function):
             # nothing is kept for a backward that cannot happen (no input wants a gradient)
             msave = _saved_rows(msum, save_percent) if any(ctx.needs_input_grad[:5]) else 0
 
-            h = torch.empty((msum, H), device=dev, dtype=torch.bfloat16)
+            # h in blocks of 32 hidden columns, [H/32][Msum][32]: the layout the down projection reads
+            h = torch.empty((H // 32, msum, 32), device=dev, dtype=torch.bfloat16)
             ab_save = torch.empty((msave, 2 * H), device=dev, dtype=torch.bfloat16) if msave > 0 else None
             _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, h, ab_save, 0, msave)
             ys = torch.empty((msum, D), device=dev, dtype=torch.bfloat16)
@@ -117,7 +118,8 @@ class MoEFunction(torch.autograd.Function):
             _hip.dgrad_h(Gy, W2, idx, table, u)
             # SwiGLU backward: rows with saved a|b read them; the others recompute a|b = x.Wl1
             # and consume them straight from the GEMM's accumulators
-            gz = torch.empty((msum, 2 * H), device=dev, dtype=torch.bfloat16)
+            # G_a|G_b in blocks of 32 columns, [2H/32][Msum][32]: the layout dL/dx contracts over
+            gz = torch.empty((2 * H // 32, msum, 32), device=dev, dtype=torch.bfloat16)
             # s*h in groups of 32 padded sorted rows, feature-major inside a group: the layout
             # the Wl2 gradient reads fastest
             hsT = torch.empty((_hip.padded_rows(msum, N) // 32, H, 32), device=dev, dtype=torch.bfloat16)
@@ -148,7 +150,7 @@ class MoEFunction(torch.autograd.Function):
             G_W1 = None
             if need_w1:
                 G_W1 = torch.empty_like(W1)
-                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, M, msum,
+                _hip.wgrad(x_MD, idx, gz, None, cumsums, G_W1, M, msum, b_kblocked=True,
                            workspace_bytes=min(ws_cap, _hip.wgrad_workspace_bytes(N, D, 2 * H, msum)))
 
             G_x_BSD = None

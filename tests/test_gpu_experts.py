@@ -133,8 +133,11 @@ def test_weight_gradient_from_a_transposed_operand(sizes, M):
             T[:, p0:p0 + n] = rows[c[e]:c[e + 1]].T
         return T.reshape(F, mpad // 32, 32).permute(1, 0, 2).contiguous()
 
+    # k-blocked B: [feature / 32, row, 32]
+    blocked_B = B.reshape(msum, Y // 32, 32).permute(1, 0, 2).contiguous()
     want = torch.stack([A[c[e]:c[e + 1]].float().T @ B[c[e]:c[e + 1]].float() for e in range(N)])
-    for kw, a, b in ((dict(a_transposed=True), grouped(A), B), (dict(b_transposed=True), A, grouped(B))):
+    for kw, a, b in ((dict(a_transposed=True), grouped(A), B), (dict(b_transposed=True), A, grouped(B)),
+                     (dict(b_kblocked=True), A, blocked_B)):
         for ws in (None, 0):
             GW = torch.full((N, X, Y), float("nan"), device=dev, dtype=torch.bfloat16)
             _hip.wgrad(a, None, b, None, cumsums, GW, M, msum, workspace_bytes=ws, **kw)
