@@ -14,6 +14,8 @@ def _logits(M, N, seed):
 @pytest.mark.parametrize("M,N,K,Ks,f32", [
     (128, 8, 2, 0, True), (8192, 128, 8, 0, True), (1000, 64, 8, 4, True),
     (513, 200, 6, 1, True), (2048, 128, 8, 0, False),
+    (77, 300, 8, 3, True),      # more than 256 experts: 8 columns per lane
+    (33, 64, 3, 0, True),       # one column per lane, a partial block of tokens
 ])
 def test_router_forward(M, N, K, Ks, f32):
     from momoe_amd import _hip
@@ -44,7 +46,9 @@ def test_router_forward(M, N, K, Ks, f32):
         torch.testing.assert_close(Ks_M.cpu(), ref["Ks_M"], rtol=1e-5, atol=1e-7)
 
 
-@pytest.mark.parametrize("M,N,K,Ks", [(256, 16, 4, 0), (1000, 64, 8, 4), (300, 130, 5, 2)])
+@pytest.mark.parametrize("M,N,K,Ks", [(256, 16, 4, 0), (1000, 64, 8, 4), (300, 130, 5, 2),
+                                      (90, 300, 8, 3),     # more than 256 experts: blocks of 16 tokens
+                                      (8192, 128, 8, 0)])  # the headline routing
 def test_router_backward(M, N, K, Ks):
     from momoe_amd import _hip
     lg = _logits(M, N, 3)
