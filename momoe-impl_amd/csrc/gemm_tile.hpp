@@ -263,17 +263,23 @@ struct TDma {
 // k-strided operand whose k-rows are the sorted rows [row_begin,row_end) of one expert,
 // optionally gathered through an index.  k-rows past row_end are pointed at the expert's last
 // row (any readable row would do): the main loop zeroes the M-side fragments of those k-values
-// in the last stage, so they add nothing.  The row ids of a deposit are a wave-uniform pair,
-// fetched with scalar loads: those of the first kFirst stages once per expert (every tile of
-// the expert starts with the same rows), the later ones one stage ahead of their use.  Sources
-// are given as a wave-uniform base plus a 32-bit byte offset per lane (the form with a full
-// 64-bit address per lane costs ~20% of the whole GEMM): the base is the matrix for a
-// gathered operand and the expert's first row otherwise, so (number of tokens) x (row pitch)
-// must stay below 4 GiB.
-struct TGatherDma {
+// in the last stage, so they add nothing.  The four row ids of a wave's deposits are
+// wave-uniform and come through scalar loads: those of the first kFirst stages once per expert
+// (every tile of the expert starts with the same rows), the later ones one stage ahead of their
+// use.  Asking for the ids (request) and turning them into offsets (resolve) are separate steps
+// a stage apart: done in one step, every wave sat out one scalar-load latency per stage right
+// after the barrier, before its transfers went out.  Sources are given as a wave-uniform base
+// plus a 32-bit byte offset per lane (the form with a full 64-bit address per lane costs ~20% of
+// the whole GEMM): the base is the matrix for a gathered operand and the expert's first row
+// otherwise, so (number of tokens) x (row pitch) must stay below 4 GiB.
+// MAY_GATHER = false: the rows are never gathered and no ids are loaded.
+template <bool MAY_GATHER>
+struct TGatherDmaT {
   using L = TLayout;
   static constexpr int NCH = L::NCH;
   static constexpr int LDS_ELEMS = L::LDS_ELEMS;
+  static constexpr int kRows = 2 * NCH;  // k-rows of one wave's deposits in a stage
+  static_assert(NCH == 2, "a wave's deposits of one stage cover four consecutive rows");
   const bf16* mat;  // wave-uniform
   uint32_t ldb;     // bytes between rows
   const int32_t* gather;
@@ -282,32 +288,33 @@ struct TGatherDma {
   struct Offs {
     uint32_t a[NCH], b[NCH];  // byte offsets of the two k-rows of each deposit
   };
+  struct Ids {
+    int32_t v[kRows];
+  };
   Offs head0, head1, head2;  // this wave's k-rows in the first three stages
-  Offs next;                 // for the next issue() call
+  Ids next;                  // ids requested for the next issue() call
   static_assert(kFirst == 3, "three cached stages");
 
-  __device__ __forceinline__ Offs row_pairs(int kt) const {
-    static_assert(NCH == 2, "a wave's deposits of one stage cover four consecutive rows");
+  // sorted row behind k-row j of this wave's deposits in stage kt
+  __device__ __forceinline__ int row_of(int kt, int j) const {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r0 = row_begin + kt * kBK + w * (2 * NCH);
-    Offs out;
-    if (gather != nullptr && r0 + 3 < row_end) {
-      // the four row ids sit next to each other: one scalar load instead of four
-      typedef int32_t i32x4 __attribute__((ext_vector_type(4), aligned(4)));
-      const i32x4 v = *(const i32x4 __attribute__((address_space(4)))*)(gather + r0);
-      out.a[0] = (uint32_t)v[0] * ldb;
-      out.b[0] = (uint32_t)v[1] * ldb;
-      out.a[1] = (uint32_t)v[2] * ldb;
-      out.b[1] = (uint32_t)v[3] * ldb;
-      return out;
-    }
+    return min(row_begin + kt * kBK + w * kRows + j, row_end - 1);
+  }
+  // start the scalar loads of the ids of stage kt; the results must not be touched before
+  // resolve()
+  __device__ __forceinline__ void request(int kt, Ids& ids) const {
+    if (!MAY_GATHER || gather == nullptr) return;  // kernel-uniform
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int ra = min(r0 + j * 2, row_end - 1);
-      const int rb = min(ra + 1, row_end - 1);
-      out.a[j] = (uint32_t)(gather ? load_uniform(gather + ra) : ra - row_begin) * ldb;
-      out.b[j] = (uint32_t)(gather ? load_uniform(gather + rb) : rb - row_begin) * ldb;
-    }
+    for (int j = 0; j < kRows; ++j) ids.v[j] = load_uniform(gather + row_of(kt, j));
+  }
+  __device__ __forceinline__ Offs resolve(int kt, const Ids& ids) const {
+    uint32_t o[kRows];
+#pragma unroll
+    for (int j = 0; j < kRows; ++j)
+      o[j] = (uint32_t)(MAY_GATHER && gather != nullptr ? ids.v[j] : row_of(kt, j) - row_begin) * ldb;
+    Offs out;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) out.a[j] = o[2 * j], out.b[j] = o[2 * j + 1];
     return out;
   }
   // once per expert (re > rb); ld_ = elements between rows of the matrix
@@ -316,9 +323,14 @@ struct TGatherDma {
     ldb = (uint32_t)(ld_ * 2);
     row_begin = rb;
     row_end = re;
-    head0 = row_pairs(0);
-    head1 = row_pairs(1);
-    head2 = row_pairs(2);
+    Ids i0, i1, i2;  // all three in flight before the first is used
+    request(0, i0);
+    request(1, i1);
+    request(2, i2);
+    __builtin_amdgcn_sched_barrier(0);
+    head0 = resolve(0, i0);
+    head1 = resolve(1, i1);
+    head2 = resolve(2, i2);
   }
   // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
   __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
@@ -336,23 +348,25 @@ struct TGatherDma {
     for (int j = 0; j < NCH; ++j)
       dma16(mat, (upper ? v.b[j] : v.a[j]) + colb[j], L::deposit(stage, j));
   }
-  // stage S < kFirst of a tile; the last of them starts the fetch for issue(kFirst)
+  // stage S < kFirst of a tile; the last of them asks for the ids of issue(kFirst)
   template <int S>
   __device__ __forceinline__ void issue_head(uint32_t stage) {
     deposit(S == 0 ? head0 : S == 1 ? head1 : head2, stage);
-    if (S == kFirst - 1) next = row_pairs(kFirst);
+    if (S == kFirst - 1) request(kFirst, next);
   }
-  // must be called with kt = kFirst, kFirst+1, ... in order: uses the offsets fetched for kt
-  // and starts fetching those of kt+1
+  // must be called with kt = kFirst, kFirst+1, ... in order: uses the ids requested for kt (a
+  // stage ago: they have long arrived) and asks for those of kt+1 only after that
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
-    const Offs cur = next;
-    next = row_pairs(kt + 1);
+    const Offs cur = resolve(kt, next);
+    __builtin_amdgcn_sched_barrier(0);
+    request(kt + 1, next);
     deposit(cur, stage);
   }
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
     return L::frag(stage, c0, kk);
   }
 };
+using TGatherDma = TGatherDmaT<true>;
 
 // ---- the k-loop -----------------------------------------------------------------------------
 // Ring of kStages LDS stage buffers; `head` is the buffer of stage 0 of the current tile and

@@ -41,7 +41,7 @@ struct RowsOperand : TGatherDma {
 // the SwiGLU backward writes it for dL/dx).  Rows are the contraction index, as in the row layout,
 // and go through the same transposing LDS reads; the 32 rows x 32 features of a block are 2 KiB
 // of consecutive memory.
-struct BlockedRowsOperand : TGatherDma {
+struct BlockedRowsOperand : TGatherDmaT<false> {
   int64_t nrows;
   __device__ __forceinline__ void begin_piece(const int32_t*, int64_t ld_, int rb, int re, int) {
     nrows = ld_;
