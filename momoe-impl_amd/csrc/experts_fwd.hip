@@ -160,18 +160,19 @@ struct Lin1Prog {
       float gsum = 0.0f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const bool incol = j0 + acc_col(q) < H;
         float va[4], vb[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float a = acc[0][i][4 * q + e], b = acc[1][i][4 * q + e];
           const float u = (float)uq[q][e];
           const float sg = sigmoidf_fast(b);
-          const float hval = a * b * sg;
-          gsum += incol ? u * hval : 0.0f;
+          const float t = b * sg;  // silu(b)
+          const float hval = a * t;
+          gsum += u * hval;
           const float gh = sv * u;
-          va[e] = gh * b * sg;
-          vb[e] = gh * a * sg * (1.0f + b * (1.0f - sg));
+          va[e] = gh * t;
+          // d silu / d b = sg (1 + b (1 - sg)) = sg + t - t sg
+          vb[e] = (gh * a) * __builtin_fmaf(-t, sg, sg + t);
           acc[0][i][4 * q + e] = sv * hval;  // a is not needed any more: keep hs in its place
         }
         stager.put(0, q, pack_bf16x4(va[0], va[1], va[2], va[3]));
@@ -219,7 +220,8 @@ struct Lin1Prog {
             *(bf16x8*)(p.hst + ((int64_t)((tc.prow0 + rl0) >> 5) * p.ldt + j0 + col) * 32 + rg * 8) = v;
         }
       }
-      gsums[i] = rl0 + acc_row() < tc.rows ? gsum : 0.0f;
+      // the wave's 32 hidden columns lie inside H or outside as a whole (H is a multiple of 32)
+      gsums[i] = rl0 + acc_row() < tc.rows && j0 < H ? gsum : 0.0f;
     }
     // every wave is done with its staging area before the row sums overwrite it
     wait_lgkm0();

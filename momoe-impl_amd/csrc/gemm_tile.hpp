@@ -291,9 +291,8 @@ struct TGatherDmaT {
   struct Ids {
     int32_t v[kRows];
   };
-  Offs head0, head1, head2;  // this wave's k-rows in the first three stages
-  Ids next;                  // ids requested for the next issue() call
-  static_assert(kFirst == 3, "three cached stages");
+  Offs head[kFirst];  // this wave's k-rows in the first stages of a tile
+  Ids next;           // ids requested for the next issue() call
 
   // sorted row behind k-row j of this wave's deposits in stage kt
   __device__ __forceinline__ int row_of(int kt, int j) const {
@@ -323,14 +322,12 @@ struct TGatherDmaT {
     ldb = (uint32_t)(ld_ * 2);
     row_begin = rb;
     row_end = re;
-    Ids i0, i1, i2;  // all three in flight before the first is used
-    request(0, i0);
-    request(1, i1);
-    request(2, i2);
+    Ids first[kFirst];  // all in flight before the first is used
+#pragma unroll
+    for (int s = 0; s < kFirst; ++s) request(s, first[s]);
     __builtin_amdgcn_sched_barrier(0);
-    head0 = resolve(0, i0);
-    head1 = resolve(1, i1);
-    head2 = resolve(2, i2);
+#pragma unroll
+    for (int s = 0; s < kFirst; ++s) head[s] = resolve(s, first[s]);
   }
   // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
   __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
@@ -351,7 +348,7 @@ struct TGatherDmaT {
   // stage S < kFirst of a tile; the last of them asks for the ids of issue(kFirst)
   template <int S>
   __device__ __forceinline__ void issue_head(uint32_t stage) {
-    deposit(S == 0 ? head0 : S == 1 ? head1 : head2, stage);
+    deposit(head[S], stage);
     if (S == kFirst - 1) request(kFirst, next);
   }
   // must be called with kt = kFirst, kFirst+1, ... in order: uses the ids requested for kt (a
@@ -408,10 +405,15 @@ __device__ __forceinline__ void gemm_issue_head(AOp& A, BOp& B, StageRing<AOp, B
 template <class AOp, class BOp>
 __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp>& ring,
                                                  int ktiles) {
-  static_assert(kFirst == 3, "written for three stages ahead");
+  static_assert(kFirst >= 2 && kFirst <= 4 && kFirst < kStages + 1, "stages requested ahead");
   gemm_issue_head<0>(A, B, ring);
   if (ktiles > 1) gemm_issue_head<1>(A, B, ring);
-  if (ktiles > 2) gemm_issue_head<2>(A, B, ring);
+  if constexpr (kFirst > 2) {
+    if (ktiles > 2) gemm_issue_head<2>(A, B, ring);
+  }
+  if constexpr (kFirst > 3) {
+    if (ktiles > 3) gemm_issue_head<3>(A, B, ring);
+  }
 }
 
 // Waits on the transfers count operations: loads of a wave complete in the order they were
@@ -421,9 +423,9 @@ __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, 
 template <int LOADS>
 __device__ __forceinline__ void wait_first_stage(int ktiles) {
   static_assert((kFirst - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
-  static_assert(kFirst == 3 || kFirst == 4, "wait ladder written for 3 or 4 stages ahead");
-  if (kFirst == 4 && ktiles > 3) wait_vmcnt<3 * LOADS>();
-  else if (ktiles > 2) wait_vmcnt<2 * LOADS>();
+  static_assert(kFirst >= 2 && kFirst <= 4, "wait ladder written for 2 to 4 stages ahead");
+  if (kFirst >= 4 && ktiles > 3) wait_vmcnt<3 * LOADS>();
+  else if (kFirst >= 3 && ktiles > 2) wait_vmcnt<2 * LOADS>();
   else if (ktiles > 1) wait_vmcnt<LOADS>();
   else wait_vmcnt<0>();
 }
@@ -432,9 +434,9 @@ __device__ __forceinline__ void wait_first_stage(int ktiles) {
 template <int LOADS>
 __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
   static_assert((kStages - 2) * LOADS <= 63, "vmcnt is a 6-bit counter");
-  static_assert(kStages == 4 || kStages == 5, "wait ladder written for 4 or 5 stages");
-  if (kStages == 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS>();
-  else if (kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
+  static_assert(kStages >= 3 && kStages <= 5, "wait ladder written for 3 to 5 stages");
+  if (kStages >= 5 && kt + 3 < ktiles) wait_vmcnt<3 * LOADS>();
+  else if (kStages >= 4 && kt + 2 < ktiles) wait_vmcnt<2 * LOADS>();
   else if (kt + 1 < ktiles) wait_vmcnt<LOADS>();
   else wait_vmcnt<0>();
 }
