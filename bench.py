@@ -30,13 +30,13 @@ PEAK_HBM_GBS = 8000.0
 # for a kernel that has not been measured.
 TRAFFIC_SOURCE = "profiles/momoe_layer_headline_fetch_size.txt + _write_size.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "momoe_lin1_swiglu_fwd": 2 * 817820 * 1024 + 137218 * 1024,
-    "momoe_lin2_scale_fwd": 2 * 401739 * 1024 + 262144 * 1024,
-    "momoe_dgrad_h": 2 * 463923 * 1024 + 131072 * 1024,
-    "momoe_lin1_swiglu_bwd": 2 * 953104 * 1024 + 406448 * 1024,
-    "momoe_wgrad[Wl2]": 2 * 216403 * 1024 + 524359 * 1024,
-    "momoe_wgrad[Wl1]": 2 * 291539 * 1024 + 1048635 * 1024,
-    "momoe_dgrad_x": 2 * 795805 * 1024 + 262144 * 1024,
+    "momoe_lin1_swiglu_fwd": 2 * 808836 * 1024 + 137116 * 1024,
+    "momoe_lin2_scale_fwd": 2 * 398250 * 1024 + 262144 * 1024,
+    "momoe_dgrad_h": 2 * 458030 * 1024 + 131072 * 1024,
+    "momoe_lin1_swiglu_bwd": 2 * 919950 * 1024 + 402739 * 1024,
+    "momoe_wgrad[Wl2]": 2 * 239251 * 1024 + 524372 * 1024,
+    "momoe_wgrad[Wl1]": 2 * 294344 * 1024 + 1048628 * 1024,
+    "momoe_dgrad_x": 2 * 795830 * 1024 + 262144 * 1024,
 }
 
 
