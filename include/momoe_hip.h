@@ -35,8 +35,14 @@ extern "C" {
 #define MOMOE_ERR_UNSUPPORTED 2 /* shape outside what the kernels handle */
 #define MOMOE_ERR_LAUNCH 3      /* the HIP runtime refused a launch */
 
-/* rows per row-tile of the grouped GEMMs; the tile table must be built with it */
-#define MOMOE_TILE_ROWS 256
+/* Rows per row tile of the grouped GEMMs.  A tile table is built for one tile height
+ * (momoe_index_build, momoe_tile_table_build).  momoe_lin1_swiglu_fwd, momoe_lin2_scale_fwd,
+ * momoe_dgrad_h and momoe_dgrad_x take tables of any height up to MOMOE_TILE_ROWS and are
+ * fastest at exactly that; momoe_lin1_swiglu_bwd takes heights up to MOMOE_RECOMPUTE_TILE_ROWS
+ * (its epilogue leaves no registers for a taller tile).  A kernel given a table of a greater
+ * height than it takes returns without writing anything. */
+#define MOMOE_TILE_ROWS 320
+#define MOMOE_RECOMPUTE_TILE_ROWS 256
 /* column-block width of the partial row sums written by momoe_lin1_swiglu_bwd */
 #define MOMOE_GS_BLOCK 128
 
@@ -77,6 +83,14 @@ int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m
                       int32_t* tile_table, int tile_rows,
                       void* workspace, int64_t workspace_bytes,
                       int32_t* violations, void* stream);
+
+/* A tile table for another tile height, from the prefix sums of a finished momoe_index_build
+ * (no counterpart in the reference: its launchers size their grids on the host).  Msum = M*K, the
+ * rows the sorted matrices were allocated for; tile_table int32[momoe_tile_table_ints(M, N, K,
+ * tile_rows)].  Same contents as the table momoe_index_build writes for that tile_rows.
+ */
+int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int64_t Msum, int tile_rows,
+                           int32_t* tile_table, void* stream);
 
 /* momoe_index_build_static: momoe_index_build without the workspace arguments, for callers
  * that cannot allocate device memory (code under HIP graph capture, tight serving loops,

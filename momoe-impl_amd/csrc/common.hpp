@@ -39,7 +39,7 @@ struct TileCoord {
   int rows;    // valid rows in this tile (1..rows per tile)
   int tn;      // column block
   int mbase;   // first tile row owned by this wave (waves 0-3 / 4-7 split the tile's rows)
-  int na;      // 32-row fragment rows owned by this wave (0..4)
+  int na;      // 32-row fragment rows owned by this wave (0..5)
   bool valid;
 };
 
@@ -60,11 +60,13 @@ struct TileSched {
   const int* table;
   int nb, bm, begin, total, chunk, xcd, pos, stride;
 
-  // tiles before row tile `first_row_tile` (all its column blocks) are left out
-  __device__ __forceinline__ TileSched(const int* table_, int nb_, int first_row_tile = 0)
+  // tiles before row tile `first_row_tile` (all its column blocks) are left out; a table whose
+  // tiles are taller than the kernel's `max_tile_rows` yields no tiles at all
+  __device__ __forceinline__ TileSched(const int* table_, int nb_, int max_tile_rows,
+                                       int first_row_tile = 0)
       : table(table_), nb(nb_) {
-    const int ntiles = *(const int __attribute__((address_space(4)))*)table;
     bm = *(const int __attribute__((address_space(4)))*)(table + 1);
+    const int ntiles = bm <= max_tile_rows ? *(const int __attribute__((address_space(4)))*)table : 0;
     begin = min(first_row_tile, ntiles) * nb;
     total = ntiles * nb;
     chunk = (total - begin + 7) >> 3;

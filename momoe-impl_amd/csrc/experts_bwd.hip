@@ -7,14 +7,16 @@
 namespace momoe {
 namespace {
 
-constexpr int BM = MOMOE_TILE_ROWS;
+using G = TallTiles;  // both data-gradient GEMMs take row tiles of up to 320 rows
 constexpr int BN = 256;
-constexpr int FM = 4, FN = 2;  // 2x4 waves, each 128 rows x 64 columns
-using RowsA = RDma<BM>;  // sorted / gathered token rows, k-contiguous
-using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
-using BlockedA = RBlockedDma<BM>;  // sorted rows of a k-blocked intermediate (gz)
-using Ring = StageRing<RowsA, RowsB>;
-constexpr size_t kBwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+constexpr int FM = G::FM, FN = G::FN;  // 2x4 waves, each 160 rows x 64 columns
+using RowsA = RDma<G::AROWS>;  // sorted / gathered token rows, k-contiguous
+using RowsB = RDma<BN>;        // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
+using BlockedA = RBlockedDma<G::AROWS>;  // sorted rows of a k-blocked intermediate (gz)
+using DhRing = StageRing<RowsA, RowsB, G::STAGES>;
+using DxRing = StageRing<BlockedA, RowsB, G::STAGES>;
+static_assert(DhRing::BYTES == DxRing::BYTES, "same stage sizes");
+constexpr size_t kBwdLds = DhRing::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
 
 struct DhArgs {
   const bf16* gy;
@@ -70,11 +72,11 @@ struct DhProg {
 
 __global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
   const ClockTrace trace(p.clk);
-  Ring ring(dyn_lds());
-  TileSched sched(p.table, (p.H + BN - 1) / BN);
+  DhRing ring(dyn_lds());
+  TileSched sched(p.table, (p.H + BN - 1) / BN, G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DhProg prog{p, p.D / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  DhProg prog{p, p.D / kBK, wn, RowStager<2>(dyn_lds() + DhRing::STAGES * DhRing::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
   trace.finish();
 }
@@ -232,11 +234,11 @@ struct DxProg {
 
 __global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
   const ClockTrace trace(p.clk);
-  StageRing<BlockedA, RowsB> ring(dyn_lds());
-  TileSched sched(p.table, (p.D + BN - 1) / BN);
+  DxRing ring(dyn_lds());
+  TileSched sched(p.table, (p.D + BN - 1) / BN, G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DxProg prog{p, (2 * p.H) / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
+  DxProg prog{p, (2 * p.H) / kBK, wn, RowStager<2>(dyn_lds() + DxRing::STAGES * DxRing::STAGE)};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
   trace.finish();
 }

@@ -1,18 +1,15 @@
 // Forward of the experts: grouped GEMM x.Wl1 with fused SwiGLU, grouped GEMM
 // h.Wl2 with the gate weight fused into the epilogue, and the K-way combine.
+#include <type_traits>
+
 #include "gemm_tile.hpp"
 
 namespace momoe {
 namespace {
 
-constexpr int BM = MOMOE_TILE_ROWS;  // 256 sorted rows per tile
-constexpr int BN = 256;              // GEMM columns per tile
-constexpr int FM = 4, FN = 2;        // 2x4 waves, each 128 rows x 64 columns
-using RowsOp = RDma<BM>;             // token rows, k-contiguous
-using HRowsOp = RBlockedDma<BM>;     // rows of h, k-blocked
-using WeightOp = TDma;               // expert weights [k][col], k-strided
-using Ring = StageRing<RowsOp, WeightOp>;
-constexpr size_t kFwdLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+constexpr int BN = 256;  // GEMM columns per tile
+constexpr int FN = 2;    // 2x4 waves, each (32 * FM) rows x 64 columns
+using WeightOp = TDma;   // expert weights [k][col], k-strided
 
 struct Lin1Args {
   const bf16* x;
@@ -35,12 +32,19 @@ struct Lin1Args {
   unsigned long long* clk;
 };
 
-// Tile = 256 rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
+// Tile = up to 320 (256) rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
 // columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
 // BWD = false: forward / recomputation, writes h and/or a|b.  BWD = true: the a|b of the tile
 // stay in registers and go straight into the SwiGLU backward.
 template <bool BWD>
 struct Lin1Prog {
+  // the forward takes tall tiles; the backward's epilogue needs the registers of the fifth
+  // fragment row, so it runs on a tile table of its own with 256-row tiles
+  using G = std::conditional_t<BWD, StdTiles, TallTiles>;
+  static constexpr int FM = G::FM, BM = G::MAX_ROWS;
+  using RowsOp = RDma<G::AROWS>;  // token rows, k-contiguous
+  using Ring = StageRing<RowsOp, WeightOp, G::STAGES>;
+  static constexpr size_t kLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
   static constexpr int BNH = BN / 2;
   static_assert(BNH == MOMOE_GS_BLOCK, "gs_part blocks follow the hidden-column tile");
   static_assert(4 * BM * sizeof(float) <= kEpilogueLds, "the dL/ds row sums reuse the staging area");
@@ -246,15 +250,17 @@ struct Lin1Prog {
 template <bool BWD>
 __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   using Prog = Lin1Prog<BWD>;
+  using Ring = typename Prog::Ring;
+  constexpr int FM = Prog::FM;
   const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   // without an h output only rows >= ab_lo are wanted: experts entirely below are skipped
   const int first_tile =
       p.h == nullptr && p.ab_lo > 0 ? TileSched::expert_tile_of_row(p.table, p.ab_lo) : 0;
-  TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, first_tile);
+  TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, Prog::BM, first_tile);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
-  Prog prog{p, p.D / kBK, wn, dyn_lds() + kStages * Ring::STAGE};
+  Prog prog{p, p.D / kBK, wn, dyn_lds() + Ring::STAGES * Ring::STAGE};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
   trace.finish();
 }
@@ -273,6 +279,11 @@ struct Lin2Args {
 };
 
 struct Lin2Prog {
+  using G = TallTiles;
+  static constexpr int FM = G::FM;
+  using HRowsOp = RBlockedDma<G::AROWS>;  // rows of h, k-blocked
+  using Ring = StageRing<HRowsOp, WeightOp, G::STAGES>;
+  static constexpr size_t kLds = Ring::BYTES + kEpilogueLds;
   struct Prep {
     int32_t tok[FM];  // tokens of the rows this lane holds in the accumulators
     float sv[FM];     // their gate weights
@@ -319,13 +330,14 @@ struct Lin2Prog {
 };
 
 __global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
+  using Ring = Lin2Prog::Ring;
   const ClockTrace trace(p.clk);
-  StageRing<HRowsOp, WeightOp> ring(dyn_lds());
-  TileSched sched(p.table, (p.D + BN - 1) / BN);
+  Ring ring(dyn_lds());
+  TileSched sched(p.table, (p.D + BN - 1) / BN, Lin2Prog::G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  Lin2Prog prog{p, p.H / kBK, wn, RowStager<2>(dyn_lds() + kStages * Ring::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  Lin2Prog prog{p, p.H / kBK, wn, RowStager<2>(dyn_lds() + Ring::STAGES * Ring::STAGE)};
+  run_row_tiles<Lin2Prog::FM, FN>(prog, sched, ring, n_org);
   trace.finish();
 }
 
@@ -395,8 +407,8 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
              nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<false>, kFwdLds, once);
-  lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel<false>, Lin1Prog<false>::kLds, once);
+  lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, Lin1Prog<false>::kLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -421,8 +433,8 @@ extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
              row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
              (bf16*)gz_blocked, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<true>, kFwdLds, once);
-  lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel<true>, Lin1Prog<true>::kLds, once);
+  lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, Lin1Prog<true>::kLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -440,8 +452,8 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_blocked, const void* Wl2_NHD, 
   Lin2Args a{(const bf16*)h_blocked, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin2_scale_kernel, kFwdLds, once);
-  lin2_scale_kernel<<<persistent_grid(), kThreads, kFwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin2_scale_kernel, Lin2Prog::kLds, once);
+  lin2_scale_kernel<<<persistent_grid(), kThreads, Lin2Prog::kLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

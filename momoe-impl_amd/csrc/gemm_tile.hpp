@@ -1,9 +1,9 @@
 // Workgroup-level bf16 GEMM building blocks for gfx950 (CDNA4).
 //
 // A workgroup of 8 wavefronts (two per SIMD: a lone wave leaves ~15% of the MFMA
-// issue slots empty) computes a 256 x 256 fp32 tile with
-// v_mfma_f32_32x32x16_bf16; each wave owns 128 x 64 of it in 8 accumulator
-// fragments (128 registers), one workgroup per CU.  Both MFMA inputs want, per lane, 8
+// issue slots empty) computes a 256 x 256 or, where registers and LDS allow, a 320 x 256 fp32
+// tile with v_mfma_f32_32x32x16_bf16; each wave owns 128 x 64 (160 x 64) of it in 8 (10)
+// accumulator fragments of 16 registers, one workgroup per CU.  Both MFMA inputs want, per lane, 8
 // consecutive k-values of one row (lane%32 = row, lane/32 = which group of 8
 // k's).  Two kinds of operand tile feed that:
 //
@@ -36,7 +36,9 @@
 //   * Rows of a ragged tile that do not exist are pointed at the last valid row: the 16
 //     lanes of a deposit then ask for one line instead of 16.  What a small tile cannot avoid
 //     is streaming its whole weight block, so an expert's rows are cut into equal row tiles
-//     rather than full tiles plus a sliver.
+//     rather than full tiles plus a sliver, and a taller tile saves whole passes over the weights:
+//     with 320-row tiles an expert of 513..640 rows takes two passes instead of three (measured
+//     -9..-11% for such experts, -10% of the bytes per flop for large ones).
 //
 // Global memory goes straight to LDS with global_load_lds_dwordx4 (no VGPR
 // staging): one wave instruction deposits 64 x 16 bytes contiguously.  Since
@@ -47,12 +49,12 @@
 // pointed at a clamped row/column (results masked at the store; along k the main loop
 // zeroes the affected fragment registers instead).
 //
-// The k-loop runs a ring of 4 stages of 32 k: while one stage is multiplied (2 MFMA
-// k-steps) the next three are in flight; one s_barrier per stage.  The fragments of
+// The k-loop runs a ring of 3 or 4 stages of 32 k: while one stage is multiplied (2 MFMA
+// k-steps) the next two or three are in flight; one s_barrier per stage.  The fragments of
 // a stage's second k-step are read before the barrier that opens the next stage and
 // multiplied after it, so the matrix pipe stays fed while the first fragments of
-// the new stage travel from LDS.  At the end of a tile three buffers are free, so
-// the next tile's first three stages are requested before the epilogue starts.
+// the new stage travel from LDS.  At the end of a tile all buffers but one are free, so
+// the next tile's first stages are requested before the epilogue starts.
 //
 // The MFMA is issued with the N-side fragment as its first input and the M-side
 // fragment as its second, so each lane ends up holding, for ONE tile row
@@ -68,8 +70,6 @@ namespace momoe {
 
 constexpr int kBK = 32;            // k-extent of one LDS stage
 constexpr int kKSteps = kBK / 16;  // MFMA k-steps per stage
-constexpr int kStages = 4;         // LDS ring depth
-constexpr int kFirst = 3;          // stages of a tile requested ahead of its main loop
 constexpr int kChunkElems = 512;   // one wave-wide 16-byte-per-lane deposit = 1 KiB
 
 // 16 bytes per lane, global -> LDS.  `lds_wave_base` is a wave-uniform LDS byte address; lane
@@ -264,7 +264,7 @@ struct TDma {
 // optionally gathered through an index.  k-rows past row_end are pointed at the expert's last
 // row (any readable row would do): the main loop zeroes the M-side fragments of those k-values
 // in the last stage, so they add nothing.  The four row ids of a wave's deposits are
-// wave-uniform and come through scalar loads: those of the first kFirst stages once per expert
+// wave-uniform and come through scalar loads: those of the first NFIRST stages once per expert
 // (every tile of the expert starts with the same rows), the later ones one stage ahead of their
 // use.  Asking for the ids (request) and turning them into offsets (resolve) are separate steps
 // a stage apart: done in one step, every wave sat out one scalar-load latency per stage right
@@ -272,8 +272,9 @@ struct TDma {
 // plus a 32-bit byte offset per lane (the form with a full 64-bit address per lane costs ~20% of
 // the whole GEMM): the base is the matrix for a gathered operand and the expert's first row
 // otherwise, so (number of tokens) x (row pitch) must stay below 4 GiB.
-// MAY_GATHER = false: the rows are never gathered and no ids are loaded.
-template <bool MAY_GATHER>
+// MAY_GATHER = false: the rows are never gathered and no ids are loaded.  NFIRST = stages of a
+// tile that are requested ahead of its main loop (the depth of the ring it is used with, less one).
+template <bool MAY_GATHER, int NFIRST>
 struct TGatherDmaT {
   using L = TLayout;
   static constexpr int NCH = L::NCH;
@@ -291,7 +292,7 @@ struct TGatherDmaT {
   struct Ids {
     int32_t v[kRows];
   };
-  Offs head[kFirst];  // this wave's k-rows in the first stages of a tile
+  Offs head[NFIRST];  // this wave's k-rows in the first stages of a tile
   Ids next;           // ids requested for the next issue() call
 
   // sorted row behind k-row j of this wave's deposits in stage kt
@@ -322,12 +323,12 @@ struct TGatherDmaT {
     ldb = (uint32_t)(ld_ * 2);
     row_begin = rb;
     row_end = re;
-    Ids first[kFirst];  // all in flight before the first is used
+    Ids first[NFIRST];  // all in flight before the first is used
 #pragma unroll
-    for (int s = 0; s < kFirst; ++s) request(s, first[s]);
+    for (int s = 0; s < NFIRST; ++s) request(s, first[s]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int s = 0; s < kFirst; ++s) head[s] = resolve(s, first[s]);
+    for (int s = 0; s < NFIRST; ++s) head[s] = resolve(s, first[s]);
   }
   // per tile: columns [col0, col0+256) of the matrix; columns >= ncols are clamped to column 0
   __device__ __forceinline__ void set_cols(const bf16* mat_, int col0, int ncols) {
@@ -345,13 +346,14 @@ struct TGatherDmaT {
     for (int j = 0; j < NCH; ++j)
       dma16(mat, (upper ? v.b[j] : v.a[j]) + colb[j], L::deposit(stage, j));
   }
-  // stage S < kFirst of a tile; the last of them asks for the ids of issue(kFirst)
+  // stage S < NFIRST of a tile; the last of them asks for the ids of issue(NFIRST)
   template <int S>
   __device__ __forceinline__ void issue_head(uint32_t stage) {
+    static_assert(S < NFIRST, "only the first stages are cached");
     deposit(head[S], stage);
-    if (S == kFirst - 1) request(kFirst, next);
+    if (S == NFIRST - 1) request(NFIRST, next);
   }
-  // must be called with kt = kFirst, kFirst+1, ... in order: uses the ids requested for kt (a
+  // must be called with kt = NFIRST, NFIRST+1, ... in order: uses the ids requested for kt (a
   // stage ago: they have long arrived) and asks for those of kt+1 only after that
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
     const Offs cur = resolve(kt, next);
@@ -363,21 +365,27 @@ struct TGatherDmaT {
     return L::frag(stage, c0, kk);
   }
 };
-using TGatherDma = TGatherDmaT<true>;
-
 // ---- the k-loop -----------------------------------------------------------------------------
-// Ring of kStages LDS stage buffers; `head` is the buffer of stage 0 of the current tile and
-// is carried from tile to tile by a persistent workgroup.
-template <class AOp, class BOp>
+// Ring of NS LDS stage buffers; `head` is the buffer of stage 0 of the current tile and is
+// carried from tile to tile by a persistent workgroup.  FIRST = NS - 1 stages of a tile are
+// requested ahead of its main loop (during the previous tile's epilogue).  Four buffers where the
+// weights stream k-row by k-row from HBM (three stages in flight cover that latency); three are
+// enough, and leave room for taller row tiles, where every line is fetched in two halves one
+// stage apart or is re-read from L2.
+template <class AOp, class BOp, int NS>
 struct StageRing {
+  static_assert(NS >= 3 && NS <= 5, "ring depth");
+  using A = AOp;
+  using B = BOp;
+  static constexpr int STAGES = NS, FIRST = NS - 1;
   static constexpr int STAGE = AOp::LDS_ELEMS + BOp::LDS_ELEMS;
-  static constexpr size_t BYTES = (size_t)kStages * STAGE * sizeof(bf16);
+  static constexpr size_t BYTES = (size_t)NS * STAGE * sizeof(bf16);
   bf16* lds;
   uint32_t addr;  // LDS byte address of `lds`
   int head;
   __device__ __forceinline__ explicit StageRing(bf16* lds_) : lds(lds_), addr(lds_address(lds_)), head(0) {}
   static __device__ __forceinline__ int slot(int s) {
-    return (kStages & (kStages - 1)) == 0 ? s & (kStages - 1) : (int)((unsigned)s % (unsigned)kStages);
+    return (NS & (NS - 1)) == 0 ? s & (NS - 1) : (int)((unsigned)s % (unsigned)NS);
   }
   __device__ __forceinline__ bf16* buf(int kt) const { return lds + slot(kt + head) * STAGE; }
   __device__ __forceinline__ uint32_t buf_addr(int kt) const {
@@ -386,26 +394,26 @@ struct StageRing {
   __device__ __forceinline__ void advance(int ktiles) { head = slot(head + ktiles); }
 };
 
-template <class AOp, class BOp>
-__device__ __forceinline__ void gemm_issue(AOp& A, BOp& B, StageRing<AOp, BOp>& ring, int kt) {
+template <class AOp, class BOp, int NS>
+__device__ __forceinline__ void gemm_issue(AOp& A, BOp& B, StageRing<AOp, BOp, NS>& ring, int kt) {
   const uint32_t st = ring.buf_addr(kt);
   A.issue(kt, st);
   B.issue(kt, st + AOp::LDS_ELEMS * 2);
 }
 
-// Request the first kFirst stages of a tile.  May be called right after the previous tile's
+// Request the first stages of a tile.  May be called right after the previous tile's
 // main loop, while other waves still multiply its last stage: the other buffers were
 // released by that tile's last barrier.
-template <int S, class AOp, class BOp>
-__device__ __forceinline__ void gemm_issue_head(AOp& A, BOp& B, StageRing<AOp, BOp>& ring) {
+template <int S, class AOp, class BOp, int NS>
+__device__ __forceinline__ void gemm_issue_head(AOp& A, BOp& B, StageRing<AOp, BOp, NS>& ring) {
   const uint32_t st = ring.buf_addr(S);
   A.template issue_head<S>(st);
   B.template issue_head<S>(st + AOp::LDS_ELEMS * 2);
 }
-template <class AOp, class BOp>
-__device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp>& ring,
+template <class AOp, class BOp, int NS>
+__device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, BOp, NS>& ring,
                                                  int ktiles) {
-  static_assert(kFirst >= 2 && kFirst <= 4 && kFirst < kStages + 1, "stages requested ahead");
+  constexpr int kFirst = NS - 1;
   gemm_issue_head<0>(A, B, ring);
   if (ktiles > 1) gemm_issue_head<1>(A, B, ring);
   if constexpr (kFirst > 2) {
@@ -420,7 +428,7 @@ __device__ __forceinline__ void gemm_issue_first(AOp& A, BOp& B, StageRing<AOp, 
 // issued, so "at most n outstanding" means "all loads but the youngest n are done" (stores that
 // are still in flight only make the wait longer).  Each wait allows exactly the stages known
 // to have been requested after the one that is needed.
-template <int LOADS>
+template <int LOADS, int kFirst>
 __device__ __forceinline__ void wait_first_stage(int ktiles) {
   static_assert((kFirst - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
   static_assert(kFirst >= 2 && kFirst <= 4, "wait ladder written for 2 to 4 stages ahead");
@@ -431,7 +439,7 @@ __device__ __forceinline__ void wait_first_stage(int ktiles) {
 }
 // wait until the deposits of stage kt (>= 1) have landed, when the stages up to kt+kStages-2
 // have been requested and everything older than stage kt is known to be complete
-template <int LOADS>
+template <int LOADS, int kStages>
 __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
   static_assert((kStages - 2) * LOADS <= 63, "vmcnt is a 6-bit counter");
   static_assert(kStages >= 3 && kStages <= 5, "wait ladder written for 3 to 5 stages");
@@ -441,8 +449,8 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
   else wait_vmcnt<0>();
 }
 
-// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.  The first kFirst
-// stages must already have been requested with gemm_issue_first.  NA is the number of 32-row
+// acc[fn][fm] += Bfrag[fn] x Afrag[fm] over `ktiles` (>= 1) stages of kBK.  The first stages
+// must already have been requested with gemm_issue_first.  NA is the number of 32-row
 // fragment rows of this wave that hold valid rows (wave-uniform): the others are neither read
 // nor multiplied; with NA = 0 the wave only takes part in the transfers and barriers.
 // `ktail` (1..kBK) is the number of k-values of the last stage that exist.
@@ -450,10 +458,11 @@ __device__ __forceinline__ void wait_stage(int kt, int ktiles) {
 // under the whole main loop (they enter the vmcnt queue between two stages, which can only
 // make the stage waits err on the long side).  On return the ring has advanced to the next
 // tile; all buffers but the last stage's are free, other waves may still be reading that one.
-template <class AOp, class BOp, int FM, int FN, int NA, class Hook>
+template <class AOp, class BOp, int NS, int FM, int FN, int NA, class Hook>
 __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
-                                              StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
+                                              StageRing<AOp, BOp, NS>& ring, const int (&m_org)[FM],
                                               const int (&n_org)[FN], Hook hook, int ktail = kBK) {
+  constexpr int kStages = NS, kFirst = NS - 1;
   static_assert(kKSteps == 2, "written for 2 k-steps per stage");
   static_assert(NA >= 0 && NA <= FM, "active fragment rows");
   constexpr int LOADS = AOp::NCH + BOp::NCH;
@@ -478,7 +487,7 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
 
   // Stage 0 has landed (the previous tile's stores need not have); every wave is done reading
   // the previous tile, whose last buffer the next stage will reuse.
-  wait_first_stage<LOADS>(ktiles);
+  wait_first_stage<LOADS, kFirst>(ktiles);
   wait_lgkm0();
   __builtin_amdgcn_s_barrier();
   fence();
@@ -497,7 +506,7 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
     fence();
     // stage kt+1 has landed; all LDS reads of stage kt have returned, so its buffer may be
     // overwritten once every wave is past the barrier
-    wait_stage<LOADS>(kt + 1, ktiles);
+    wait_stage<LOADS, kStages>(kt + 1, ktiles);
     wait_lgkm0();
     __builtin_amdgcn_s_barrier();
     fence();
@@ -532,18 +541,42 @@ __device__ __forceinline__ void gemm_mainloop(AOp& A, BOp& B, f32x16 (&acc)[FN][
   ring.advance(ktiles);
 }
 
+// Row-tile geometry of a kernel: two wave rows of FM 32-row fragment rows each (tiles of up to
+// 64 * FM rows, 64 columns per wave), the rows of the row operand's stage buffer (whole deposits
+// of 16 rows per wave, so a multiple of 128 that holds the tallest tile) and the ring depth.
+template <int FM_, int NS_>
+struct RowTileGeometry {
+  static constexpr int FM = FM_, FN = 2;
+  static constexpr int MAX_ROWS = 64 * FM;
+  static constexpr int AROWS = (MAX_ROWS + 127) / 128 * 128;
+  static constexpr int STAGES = NS_;
+};
+// 256-row tiles with a 4-stage ring: the kernel whose epilogue leaves no registers for more
+using StdTiles = RowTileGeometry<4, 4>;
+// 320-row tiles: 10 accumulator fragments per wave, a 384-row stage buffer whose last 64 rows
+// repeat the tile's last row, and a 3-stage ring to pay for it in LDS
+using TallTiles = RowTileGeometry<5, 3>;
+static_assert(TallTiles::MAX_ROWS == MOMOE_TILE_ROWS && StdTiles::MAX_ROWS == MOMOE_RECOMPUTE_TILE_ROWS,
+              "tile heights promised by the header");
+
 // main loop for a wave that owns `na` fragment rows starting at tile row m_org[0]
-template <class AOp, class BOp, int FM, int FN, class Hook>
+template <class AOp, class BOp, int NS, int FM, int FN, class Hook>
 __device__ __forceinline__ void gemm_rows(AOp& A, BOp& B, f32x16 (&acc)[FN][FM], int ktiles,
-                                          StageRing<AOp, BOp>& ring, const int (&m_org)[FM],
+                                          StageRing<AOp, BOp, NS>& ring, const int (&m_org)[FM],
                                           const int (&n_org)[FN], int na_, Hook hook) {
-  static_assert(FM == 4, "dispatch written for 4 fragment rows per wave");
+  static_assert(FM == 4 || FM == 5, "dispatch written for 4 or 5 fragment rows per wave");
   const int na = __builtin_amdgcn_readfirstlane(na_);
-  if (na == 4) gemm_mainloop<AOp, BOp, FM, FN, 4>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 3) gemm_mainloop<AOp, BOp, FM, FN, 3>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 2) gemm_mainloop<AOp, BOp, FM, FN, 2>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else if (na == 1) gemm_mainloop<AOp, BOp, FM, FN, 1>(A, B, acc, ktiles, ring, m_org, n_org, hook);
-  else gemm_mainloop<AOp, BOp, FM, FN, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  if constexpr (FM == 5) {
+    if (na == 5) {
+      gemm_mainloop<AOp, BOp, NS, FM, FN, 5>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+      return;
+    }
+  }
+  if (na == 4) gemm_mainloop<AOp, BOp, NS, FM, FN, 4>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 3) gemm_mainloop<AOp, BOp, NS, FM, FN, 3>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 2) gemm_mainloop<AOp, BOp, NS, FM, FN, 2>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else if (na == 1) gemm_mainloop<AOp, BOp, NS, FM, FN, 1>(A, B, acc, ktiles, ring, m_org, n_org, hook);
+  else gemm_mainloop<AOp, BOp, NS, FM, FN, 0>(A, B, acc, ktiles, ring, m_org, n_org, hook);
 }
 
 // the workgroup's dynamic LDS (size given at launch)
@@ -606,8 +639,8 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
 // While tile t is multiplied: the table entry of tile t+2 and the gathered values of tile t+1
 // are in flight; after its main loop the first stages of tile t+1 are requested, then the
 // epilogue of tile t runs.
-template <int FM, int FN, class P, class AOp, class BOp>
-__device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp>& ring,
+template <int FM, int FN, class P, class AOp, class BOp, int NS>
+__device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp, NS>& ring,
                                               const int (&n_org)[FN]) {
   TileCoord c0 = sched.next();
   if (!c0.valid) return;
@@ -623,8 +656,10 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
     TileSched::Raw rn;
-    const int m_org[FM] = {c0.mbase, c0.mbase + 32, c0.mbase + 64, c0.mbase + 96};
-    gemm_rows<AOp, BOp, FM, FN>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.na, [&] {
+    int m_org[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) m_org[i] = c0.mbase + 32 * i;
+    gemm_rows<AOp, BOp, NS, FM, FN>(A, B, acc, prog.ktiles, ring, m_org, n_org, c0.na, [&] {
       prog.late(c0, p0);
       if (c1.valid) prog.gather(c1, p1);
       rn = sched.fetch();

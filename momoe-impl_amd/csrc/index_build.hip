@@ -291,10 +291,61 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
   }
 }
 
+// A tile table for another tile height from the prefix sums of a finished index build.
+__global__ __launch_bounds__(1024) void tile_table_kernel(const int32_t* __restrict__ cumsums, int N,
+                                                          int64_t msum_cap, int tile_rows,
+                                                          int32_t* __restrict__ table) {
+  __shared__ int32_t s_first[kMaxExperts];
+  __shared__ int32_t s_tiles;
+  const int t = threadIdx.x, lane = t & 63;
+  if (t < 64) {
+    int run_tiles = 0;
+    for (int i0 = 0; i0 < N; i0 += 64) {
+      const int i = i0 + lane;
+      const int v = i < N ? cumsums[i + 1] - cumsums[i] : 0;
+      const int nt = (v + tile_rows - 1) / tile_rows;
+      const int inct = wave_inclusive_scan(nt, lane);
+      if (i < N) s_first[i] = run_tiles + inct - nt;
+      run_tiles += __shfl(inct, 63);
+    }
+    if (lane == 0) {
+      // an index build that found more pairs than rows emptied its table: so does this one
+      const int ntiles = (int64_t)cumsums[N] > msum_cap ? 0 : run_tiles;
+      s_tiles = ntiles;
+      table[0] = ntiles;
+      table[1] = tile_rows;
+      table[2] = 0;
+      table[3] = 0;
+    }
+  }
+  __syncthreads();
+  if (s_tiles == 0) return;
+  for (int i = t; i < N; i += 1024) {
+    const int c = cumsums[i], v = cumsums[i + 1] - c;
+    const int nt = (v + tile_rows - 1) / tile_rows;
+    const int first = s_first[i];
+    for (int k = 0; k < nt; ++k) {
+      int32_t* e = table + kTileHeader + 4 * (first + k);
+      e[0] = i;
+      e[1] = first;
+      e[2] = c;
+      e[3] = v;
+    }
+  }
+}
+
 }  // namespace
 }  // namespace momoe
 
 using namespace momoe;
+
+extern "C" int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int64_t Msum,
+                                      int tile_rows, int32_t* tile_table, void* stream) {
+  if (!cumsums_N1 || !tile_table || N <= 0 || Msum <= 0 || tile_rows <= 0) return MOMOE_ERR_BAD_ARG;
+  if (N > kMaxExperts || Msum >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(cumsums_N1, (int)N, Msum, tile_rows, tile_table);
+  return launch_status();
+}
 
 extern "C" int64_t momoe_tile_table_ints(int64_t M, int64_t N, int64_t K, int tile_rows) {
   if (M < 0 || N < 0 || K < 0 || tile_rows <= 0) return -1;

@@ -21,6 +21,7 @@ namespace {
 
 constexpr int BX = 256;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
+constexpr int kStages = 3;  // ring depth: 16 stages per tile and L2-resident operands do not need more
 constexpr int kRingBytes = kStages * 2 * TLayout::LDS_ELEMS * 2;  // every operand kind: 16 KiB per stage
 constexpr size_t kWgradLds = kRingBytes + kEpilogueLds;  // stage ring + per-wave store staging
 constexpr int kMaxWgradExperts = 4096;  // 20 bytes of prefix sums per expert fit the stage ring
@@ -31,7 +32,7 @@ static_assert(BX * BY * 4 == MOMOE_WGRAD_PARTIAL_BYTES, "size of one fp32 partia
 static_assert((size_t)(kMaxWgradExperts + 1) * 20 + 512 <= kRingBytes, "prefix sums overlay the ring");
 
 // "rows" operand of a work item: the gathered / sorted rows [rb, re)
-struct RowsOperand : TGatherDma {
+struct RowsOperand : TGatherDmaT<true, kStages - 1> {
   __device__ __forceinline__ void begin_piece(const int32_t* gather_, int64_t ld_, int rb, int re, int) {
     set_rows(gather_, ld_, rb, re);
   }
@@ -41,7 +42,7 @@ struct RowsOperand : TGatherDma {
 // the SwiGLU backward writes it for dL/dx).  Rows are the contraction index, as in the row layout,
 // and go through the same transposing LDS reads; the 32 rows x 32 features of a block are 2 KiB
 // of consecutive memory.
-struct BlockedRowsOperand : TGatherDmaT<false> {
+struct BlockedRowsOperand : TGatherDmaT<false, kStages - 1> {
   int64_t nrows;
   __device__ __forceinline__ void begin_piece(const int32_t*, int64_t ld_, int rb, int re, int) {
     nrows = ld_;
@@ -305,7 +306,7 @@ __device__ __forceinline__ f32x4* partial_piece(float* ws, int slot, int i, int 
 // an expert holds at most M rows): the bookkeeping of pieces is compiled out.
 template <bool CUT, class AOp, class BOp, int FM, int FN>
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
-  using Ring = StageRing<AOp, BOp>;
+  using Ring = StageRing<AOp, BOp, kStages>;
   static_assert(Ring::BYTES == kRingBytes, "ring size assumed by the launch");
   const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
     const int ktail = tc.re - tc.rb - (ktiles - 1) * kBK;
     const WTile nx = next_tile();
     if (ktiles > 0)
-      gemm_mainloop<AOp, BOp, FM, FN, FM>(A, B, acc, ktiles, ring, wt.m_org, wt.n_org, [] {}, ktail);
+      gemm_mainloop<AOp, BOp, kStages, FM, FN, FM>(A, B, acc, ktiles, ring, wt.m_org, wt.n_org, [] {}, ktail);
     if (nx.valid) start(nx);
 
     if (!CUT || tc.slot < 0) {

@@ -13,7 +13,8 @@ import torch  # noqa: F401  (loads the HIP runtime)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmomoe_hip.so")
 
-TILE_ROWS = 256
+TILE_ROWS = 320            # MOMOE_TILE_ROWS: tile height of the table index_build returns
+RECOMPUTE_TILE_ROWS = 256  # MOMOE_RECOMPUTE_TILE_ROWS: what lin1_swiglu_bwd takes
 GS_BLOCK = 128
 
 if not os.path.exists(LIB_PATH):
@@ -35,6 +36,7 @@ _SIGNATURES = {
     "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
     "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
                                  _p, _i64, _p, _p]),
+    "momoe_tile_table_build": (_int, [_p, _i64, _i64, _int, _p, _p]),
     "momoe_index_build_static": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p,
                                         _int, _p, _p]),
     "momoe_lin1_swiglu_fwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64,
@@ -173,6 +175,16 @@ def index_build(mask_NM, K, static_scratch=False):
               TILE_ROWS, _ptr(ws), ws_bytes, _ptr(violations), _stream())
     return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
             "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
+
+
+def tile_table_build(cumsums_N1, M, K, tile_rows):
+    """The tile table of a finished index build for another tile height (momoe_tile_table_build)."""
+    _need_cuda(cumsums_N1)
+    N = cumsums_N1.numel() - 1
+    table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, tile_rows), dtype=torch.int32,
+                        device=cumsums_N1.device)
+    _call("momoe_tile_table_build", _ptr(cumsums_N1), N, M * K, tile_rows, _ptr(table), _stream())
+    return table
 
 
 # ---------------------------------------------------------------- experts fwd

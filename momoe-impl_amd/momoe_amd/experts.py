@@ -128,7 +128,10 @@ class MoEFunction(torch.autograd.Function):
             if msave > 0:
                 _hip.swiglu_bwd_saved(ab_save, u, s, idx, cumsums, msave, gz, hsT, gs_part)
             if msave < msum:
-                _hip.lin1_swiglu_bwd(x_MD, W1, idx, table, u, s, msave, gz, hsT, gs_part)
+                # the recomputing GEMM takes shorter row tiles than the others: its own table
+                table_rc = _hip.tile_table_build(cumsums, M, ctx.K, _hip.RECOMPUTE_TILE_ROWS)
+                _hip.lin1_swiglu_bwd(x_MD, W1, idx, table_rc, u, s, msave, gz, hsT, gs_part)
+                del table_rc
             del u
 
             G_s = None

@@ -281,3 +281,30 @@ def test_input_formats_and_partial_gradients():
     with torch.no_grad():
         yn, _ = layer(xc, mask.to(dev), s.contiguous().to(dev))
     assert not yn.requires_grad and torch.equal(yn, yc.detach())
+
+
+def test_recomputing_gemm_ignores_a_table_of_taller_tiles():
+    """momoe_lin1_swiglu_bwd takes row tiles of at most 256 rows: given the 320-row table of the other
+    GEMMs it must leave its outputs alone instead of computing on tiles it cannot hold."""
+    from momoe_amd import _hip
+    M, D, H, N, K = 2048, 128, 64, 2, 1
+    x, W1, _, mask, s, _ = make_layer_inputs(M, D, H, N, K, seed=5)
+    dev = "cuda:0"
+    ib = _hip.index_build(mask.to(dev), K)
+    msum = M * K
+    assert _hip.TILE_ROWS > _hip.RECOMPUTE_TILE_ROWS and int(ib["sizes_N"].max()) > _hip.RECOMPUTE_TILE_ROWS
+    u = torch.randn(msum, H, device=dev).to(torch.bfloat16)
+    xb, W1b, sd = x.to(dev).to(torch.bfloat16), W1.to(dev), s.to(dev)
+
+    def run(table):
+        gz = torch.full((2 * H // 32, msum, 32), 7.0, device=dev, dtype=torch.bfloat16)
+        hsT = torch.full((_hip.padded_rows(msum, N) // 32, H, 32), 7.0, device=dev, dtype=torch.bfloat16)
+        gs_part = torch.full(((H + _hip.GS_BLOCK - 1) // _hip.GS_BLOCK, msum), 7.0, device=dev)
+        _hip.lin1_swiglu_bwd(xb, W1b, ib["idx_Msum"], table, u, sd, 0, gz, hsT, gs_part)
+        torch.cuda.synchronize()
+        return gz, hsT, gs_part
+
+    for t in run(ib["tile_table"]):
+        assert bool((t == 7.0).all())
+    own = _hip.tile_table_build(ib["cumsums_N"], M, K, _hip.RECOMPUTE_TILE_ROWS)
+    assert not bool((run(own)[0] == 7.0).all())

@@ -16,16 +16,10 @@ def _run(mask, K):
     return {k: v.cpu() for k, v in out.items()}
 
 
-def _compare(mask, K, out):
-    o = oracle.index_build(mask)
-    assert out["sizes_N"].dtype == torch.int64 and out["cumsums_N"].dtype == torch.int32
-    for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum"):
-        assert np.array_equal(out[k].numpy(), o[k]), k
-    assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
-    assert out["violations"].item() == 0
+def _check_table(t, o, tile_rows):
     # tile table: every expert's rows are covered exactly once, in order
-    t = out["tile_table"].numpy()
     nt, bm = int(t[0]), int(t[1])
+    assert bm == tile_rows
     ent = t[4:4 + 4 * nt].reshape(nt, 4)
     expect = []
     for i, (c0, sz) in enumerate(zip(o["cumsums_N"][:-1], o["sizes_N"])):
@@ -33,6 +27,23 @@ def _compare(mask, K, out):
         for _ in range(-(-int(sz) // bm)):
             expect.append((i, first, int(c0), int(sz)))
     assert ent.tolist() == [list(e) for e in expect]
+
+
+def _compare(mask, K, out):
+    from momoe_amd import _hip
+    o = oracle.index_build(mask)
+    assert out["sizes_N"].dtype == torch.int64 and out["cumsums_N"].dtype == torch.int32
+    for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum"):
+        assert np.array_equal(out[k].numpy(), o[k]), k
+    assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
+    assert out["violations"].item() == 0
+    _check_table(out["tile_table"].numpy(), o, _hip.TILE_ROWS)
+    # the table for another tile height, made from the prefix sums alone
+    M = mask.shape[1]
+    for rows in (_hip.RECOMPUTE_TILE_ROWS, _hip.TILE_ROWS, 32):
+        t = _hip.tile_table_build(out["cumsums_N"].to("cuda:0"), M, K, rows)
+        torch.cuda.synchronize()
+        _check_table(t.cpu().numpy(), o, rows)
 
 
 @pytest.mark.parametrize("M,N,K,Ks,skew", [
@@ -83,6 +94,10 @@ def test_violations_single_panel():
     over = torch.ones(40, 100, dtype=torch.int32)
     out = _run(over, 4)
     assert out["violations"].item() >= 1 and out["tile_table"][0].item() == 0
+    # a table made from those prefix sums is empty as well
+    from momoe_amd import _hip
+    t = _hip.tile_table_build(out["cumsums_N"].to("cuda:0"), 100, 4, _hip.RECOMPUTE_TILE_ROWS)
+    assert t[0].item() == 0
 
 
 def test_strided_mask_single_panel():
