@@ -37,10 +37,14 @@ extern "C" {
 
 /* Rows per row tile of the grouped GEMMs.  A tile table is built for one tile height
  * (momoe_index_build, momoe_tile_table_build).  momoe_lin1_swiglu_fwd, momoe_lin2_scale_fwd,
- * momoe_dgrad_h and momoe_dgrad_x take tables of any height up to MOMOE_TILE_ROWS and are
- * fastest at exactly that; momoe_lin1_swiglu_bwd takes heights up to MOMOE_RECOMPUTE_TILE_ROWS
- * (its epilogue leaves no registers for a taller tile).  A kernel given a table of a greater
- * height than it takes returns without writing anything. */
+ * momoe_dgrad_h and momoe_dgrad_x take tables of any height up to MOMOE_TILE_ROWS: they hold
+ * one code path for heights up to MOMOE_RECOMPUTE_TILE_ROWS and one for taller tiles, and follow
+ * the table.  momoe_lin1_swiglu_bwd takes heights up to MOMOE_RECOMPUTE_TILE_ROWS (its epilogue
+ * leaves no registers for a taller tile).  A kernel given a table of a greater height than it
+ * takes returns without writing anything.
+ * tile_rows = 0 in momoe_index_build lets the library choose between the two heights from the
+ * routing itself, on the device: taller tiles when they save enough passes over the experts'
+ * weights (e.g. experts of 513..640 rows: two row tiles instead of three), else the shorter. */
 #define MOMOE_TILE_ROWS 320
 #define MOMOE_RECOMPUTE_TILE_ROWS 256
 /* column-block width of the partial row sums written by momoe_lin1_swiglu_bwd */

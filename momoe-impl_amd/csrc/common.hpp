@@ -53,6 +53,10 @@ struct TileCoord {
 // fetch() issues the scalar loads of the workgroup's next tile, resolve() does the arithmetic.
 struct TileSched {
   static constexpr int kBandTiles = 4;
+  // tile height the table was built for
+  static __device__ __forceinline__ int tile_rows_of(const int* table) {
+    return *(const int __attribute__((address_space(4)))*)(table + 1);
+  }
   struct Raw {
     int q, expert, first, rstart, mi;
     bool any;

@@ -2,21 +2,17 @@
 // backward for rows whose pre-activations were saved (the others get theirs in the epilogue of
 // the recomputing x.Wl1 GEMM), dL/dx in sorted order, and the scatter of the gate-weight
 // gradient into [N, M].
+#include <algorithm>
+
 #include "gemm_tile.hpp"
 
 namespace momoe {
 namespace {
 
-using G = TallTiles;  // both data-gradient GEMMs take row tiles of up to 320 rows
+// Both data-gradient GEMMs hold both row-tile geometries and follow the tile table they are given.
 constexpr int BN = 256;
-constexpr int FM = G::FM, FN = G::FN;  // 2x4 waves, each 160 rows x 64 columns
-using RowsA = RDma<G::AROWS>;  // sorted / gathered token rows, k-contiguous
-using RowsB = RDma<BN>;        // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
-using BlockedA = RBlockedDma<G::AROWS>;  // sorted rows of a k-blocked intermediate (gz)
-using DhRing = StageRing<RowsA, RowsB, G::STAGES>;
-using DxRing = StageRing<BlockedA, RowsB, G::STAGES>;
-static_assert(DhRing::BYTES == DxRing::BYTES, "same stage sizes");
-constexpr size_t kBwdLds = DhRing::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+constexpr int FN = 2;    // 2x4 waves, each (32 * FM) rows x 64 columns
+using RowsB = RDma<BN>;  // weight rows, k-contiguous (the "NT" GEMMs of the data gradients)
 
 struct DhArgs {
   const bf16* gy;
@@ -29,13 +25,16 @@ struct DhArgs {
 };
 
 // u = G_y[idx] . Wl2^T is an "NT" GEMM: both operands are k-contiguous (k = D).
+template <class G>
 struct DhProg {
+  static constexpr int FM = G::FM;
+  using RowsA = RDma<G::AROWS>;  // gathered token rows, k-contiguous
+  using Ring = StageRing<RowsA, RowsB, G::STAGES>;  // its idle buffer is the store staging
   struct Prep {
     int32_t tok[RowsA::NCH];  // tokens of the rows this lane fetches
   };
   const DhArgs& p;
   const int ktiles, wn;
-  RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
@@ -49,8 +48,9 @@ struct DhProg {
     A.init(p.gy, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
     B.init(w, [&](int r, int) { return (uint32_t)min(n0 + r, H - 1) * (uint32_t)(2 * D); });
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&, bf16* epi) const {
     const int H = p.H;
+    const RowStager<2> stager(epi);
     const int n0 = tc.tn * BN + wn * 64;  // first hidden column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -70,16 +70,24 @@ struct DhProg {
   }
 };
 
-__global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
-  const ClockTrace trace(p.clk);
-  DhRing ring(dyn_lds());
+template <class G>
+__device__ __forceinline__ void dgrad_h_tiles(const DhArgs& p) {
+  using Prog = DhProg<G>;
+  typename Prog::Ring ring(dyn_lds());
   TileSched sched(p.table, (p.H + BN - 1) / BN, G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DhProg prog{p, p.D / kBK, wn, RowStager<2>(dyn_lds() + DhRing::STAGES * DhRing::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  Prog prog{p, p.D / kBK, wn};
+  run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);
+}
+
+__global__ __launch_bounds__(kThreads, 2) void dgrad_h_kernel(DhArgs p) {
+  const ClockTrace trace(p.clk);
+  if (TileSched::tile_rows_of(p.table) > StdTiles::MAX_ROWS) dgrad_h_tiles<TallTiles>(p);
+  else dgrad_h_tiles<StdTiles>(p);
   trace.finish();
 }
+constexpr size_t kDhLds = std::max(DhProg<TallTiles>::Ring::BYTES, DhProg<StdTiles>::Ring::BYTES);
 
 // SwiGLU backward for the sorted rows whose a|b were saved by the forward.  One workgroup per
 // group of 32 padded sorted rows (an expert's rows start at a multiple of 32 in padded
@@ -196,11 +204,14 @@ struct DxArgs {
 };
 
 // gxs = gz . Wl1^T: contraction over the 2H contiguous columns of both operands.
+template <class G>
 struct DxProg {
+  static constexpr int FM = G::FM;
+  using BlockedA = RBlockedDma<G::AROWS>;  // sorted rows of the k-blocked gz
+  using Ring = StageRing<BlockedA, RowsB, G::STAGES>;
   struct Prep {};
   const DxArgs& p;
   const int ktiles, wn;
-  RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord&, Prep&) const {}
   __device__ __forceinline__ void late(const TileCoord&, Prep&) const {}
@@ -211,8 +222,9 @@ struct DxProg {
     A.init(p.gz, p.msum, t.row0, t.rows);
     B.init(w, [&](int r, int) { return (uint32_t)min(d0 + r, D - 1) * (uint32_t)(2 * H2); });
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&) const {
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep&, bf16* epi) const {
     const int D = p.D;
+    const RowStager<2> stager(epi);
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -232,16 +244,24 @@ struct DxProg {
   }
 };
 
-__global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
-  const ClockTrace trace(p.clk);
-  DxRing ring(dyn_lds());
+template <class G>
+__device__ __forceinline__ void dgrad_x_tiles(const DxArgs& p) {
+  using Prog = DxProg<G>;
+  typename Prog::Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN, G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  DxProg prog{p, (2 * p.H) / kBK, wn, RowStager<2>(dyn_lds() + DxRing::STAGES * DxRing::STAGE)};
-  run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+  Prog prog{p, (2 * p.H) / kBK, wn};
+  run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);
+}
+
+__global__ __launch_bounds__(kThreads, 2) void dgrad_x_kernel(DxArgs p) {
+  const ClockTrace trace(p.clk);
+  if (TileSched::tile_rows_of(p.table) > StdTiles::MAX_ROWS) dgrad_x_tiles<TallTiles>(p);
+  else dgrad_x_tiles<StdTiles>(p);
   trace.finish();
 }
+constexpr size_t kDxLds = std::max(DxProg<TallTiles>::Ring::BYTES, DxProg<StdTiles>::Ring::BYTES);
 
 __global__ __launch_bounds__(256) void gs_scatter_kernel(const float* __restrict__ part, int nparts,
                                                          const int32_t* __restrict__ idx,
@@ -287,8 +307,8 @@ extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32
   DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, idx_Msum, tile_table, (bf16*)u_MsumH, (int)D,
            (int)H, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(dgrad_h_kernel, kBwdLds, once);
-  dgrad_h_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_h_kernel, kDhLds, once);
+  dgrad_h_kernel<<<persistent_grid(), kThreads, kDhLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -341,7 +361,7 @@ extern "C" int momoe_dgrad_x(const void* gz_blocked, const void* Wl1_ND2H,
   DxArgs a{(const bf16*)gz_blocked, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
            (int)H, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(dgrad_x_kernel, kBwdLds, once);
-  dgrad_x_kernel<<<persistent_grid(), kThreads, kBwdLds, (hipStream_t)stream>>>(a);
+  allow_lds(dgrad_x_kernel, kDxLds, once);
+  dgrad_x_kernel<<<persistent_grid(), kThreads, kDxLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }

@@ -1,5 +1,6 @@
 // Forward of the experts: grouped GEMM x.Wl1 with fused SwiGLU, grouped GEMM
 // h.Wl2 with the gate weight fused into the epilogue, and the K-way combine.
+#include <algorithm>
 #include <type_traits>
 
 #include "gemm_tile.hpp"
@@ -36,15 +37,15 @@ struct Lin1Args {
 // columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
 // BWD = false: forward / recomputation, writes h and/or a|b.  BWD = true: the a|b of the tile
 // stay in registers and go straight into the SwiGLU backward.
-template <bool BWD>
+// G: the row-tile geometry.  The forward takes either; the backward's epilogue needs the registers
+// of the fifth fragment row, so it only exists for 256-row tiles and runs on a tile table of its own.
+template <bool BWD, class G>
 struct Lin1Prog {
-  // the forward takes tall tiles; the backward's epilogue needs the registers of the fifth
-  // fragment row, so it runs on a tile table of its own with 256-row tiles
-  using G = std::conditional_t<BWD, StdTiles, TallTiles>;
+  static_assert(!BWD || std::is_same_v<G, StdTiles>, "the SwiGLU backward epilogue fits 256-row tiles only");
   static constexpr int FM = G::FM, BM = G::MAX_ROWS;
   using RowsOp = RDma<G::AROWS>;  // token rows, k-contiguous
   using Ring = StageRing<RowsOp, WeightOp, G::STAGES>;
-  static constexpr size_t kLds = Ring::BYTES + kEpilogueLds;  // stage ring + per-wave store staging
+  static constexpr size_t kLds = Ring::BYTES;
   static constexpr int BNH = BN / 2;
   static_assert(BNH == MOMOE_GS_BLOCK, "gs_part blocks follow the hidden-column tile");
   static_assert(4 * BM * sizeof(float) <= kEpilogueLds, "the dL/ds row sums reuse the staging area");
@@ -55,7 +56,6 @@ struct Lin1Prog {
   };
   const Lin1Args& p;
   const int ktiles, wn;
-  bf16* epi;  // store staging; in the backward also the row-sum exchange
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
@@ -78,12 +78,13 @@ struct Lin1Prog {
     A.init(p.x, [&](int, int j) { return (uint32_t)g.tok[j] * (uint32_t)(2 * D); });
     B.init(w, [&](int c) { return (c / BNH) * H + min(j0 + (c % BNH), H - 8); }, 2 * H);
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
-    if (BWD) epilogue_bwd(tc, acc, g);
-    else epilogue_fwd(tc, acc);
+  // epi: store staging; in the backward also the row-sum exchange
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g, bf16* epi) const {
+    if (BWD) epilogue_bwd(tc, acc, g, epi);
+    else epilogue_fwd(tc, acc, epi);
   }
 
-  __device__ __forceinline__ void epilogue_fwd(const TileCoord& tc, f32x16 (&acc)[FN][FM]) const {
+  __device__ __forceinline__ void epilogue_fwd(const TileCoord& tc, f32x16 (&acc)[FN][FM], bf16* epi) const {
     const int H = p.H;
     RowStager<1> stager(epi);
     const int j0 = tc.tn * BNH + wn * 32;  // first hidden column of this wave
@@ -138,7 +139,7 @@ struct Lin1Prog {
   // SwiGLU backward on the recomputed a|b (momoe/momoe.py:421-535): with u = dL/dh before the
   // gate weight s,  G_a = s u b sig(b),  G_b = s u a sig(b) (1 + b (1 - sig(b))),
   // hs = s a b sig(b),  and the partial row sum of u a b sig(b) over this tile's columns.
-  __device__ __forceinline__ void epilogue_bwd(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+  __device__ __forceinline__ void epilogue_bwd(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g, bf16* epi) const {
     const int H = p.H;
     RowStager<1> stager(epi);
     float* red = (float*)epi;  // [4 column waves][BM]
@@ -247,12 +248,11 @@ struct Lin1Prog {
   }
 };
 
-template <bool BWD>
-__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
-  using Prog = Lin1Prog<BWD>;
+template <bool BWD, class G>
+__device__ __forceinline__ void lin1_swiglu_tiles(const Lin1Args& p) {
+  using Prog = Lin1Prog<BWD, G>;
   using Ring = typename Prog::Ring;
   constexpr int FM = Prog::FM;
-  const ClockTrace trace(p.clk);
   Ring ring(dyn_lds());
   // without an h output only rows >= ab_lo are wanted: experts entirely below are skipped
   const int first_tile =
@@ -260,10 +260,24 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
   TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, Prog::BM, first_tile);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
-  Prog prog{p, p.D / kBK, wn, dyn_lds() + Ring::STAGES * Ring::STAGE};
+  Prog prog{p, p.D / kBK, wn};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
+}
+
+// The forward holds both geometries and follows the tile table it is given.
+template <bool BWD>
+__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
+  const ClockTrace trace(p.clk);
+  if constexpr (BWD) {
+    lin1_swiglu_tiles<true, StdTiles>(p);
+  } else {
+    if (TileSched::tile_rows_of(p.table) > StdTiles::MAX_ROWS) lin1_swiglu_tiles<false, TallTiles>(p);
+    else lin1_swiglu_tiles<false, StdTiles>(p);
+  }
   trace.finish();
 }
+constexpr size_t kLin1FwdLds = std::max(Lin1Prog<false, TallTiles>::kLds, Lin1Prog<false, StdTiles>::kLds);
+constexpr size_t kLin1BwdLds = Lin1Prog<true, StdTiles>::kLds;
 
 struct Lin2Args {
   const bf16* h;
@@ -278,19 +292,18 @@ struct Lin2Args {
   unsigned long long* clk;
 };
 
+template <class G>
 struct Lin2Prog {
-  using G = TallTiles;
   static constexpr int FM = G::FM;
   using HRowsOp = RBlockedDma<G::AROWS>;  // rows of h, k-blocked
   using Ring = StageRing<HRowsOp, WeightOp, G::STAGES>;
-  static constexpr size_t kLds = Ring::BYTES + kEpilogueLds;
+  static constexpr size_t kLds = Ring::BYTES;
   struct Prep {
     int32_t tok[FM];  // tokens of the rows this lane holds in the accumulators
     float sv[FM];     // their gate weights
   };
   const Lin2Args& p;
   const int ktiles, wn;
-  RowStager<2> stager;
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
@@ -307,8 +320,9 @@ struct Lin2Prog {
     A.init(p.h, p.msum, t.row0, t.rows);
     B.init(w, [&](int c) { return min(d0 + c, D - 8); }, D);
   }
-  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g) const {
+  __device__ __forceinline__ void epilogue(const TileCoord& tc, f32x16 (&acc)[FN][FM], const Prep& g, bf16* epi) const {
     const int D = p.D;
+    const RowStager<2> stager(epi);
     const int d0 = tc.tn * BN + wn * 64;  // first output column of this wave
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
@@ -329,17 +343,24 @@ struct Lin2Prog {
   }
 };
 
-__global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
-  using Ring = Lin2Prog::Ring;
-  const ClockTrace trace(p.clk);
-  Ring ring(dyn_lds());
-  TileSched sched(p.table, (p.D + BN - 1) / BN, Lin2Prog::G::MAX_ROWS);
+template <class G>
+__device__ __forceinline__ void lin2_scale_tiles(const Lin2Args& p) {
+  using Prog = Lin2Prog<G>;
+  typename Prog::Ring ring(dyn_lds());
+  TileSched sched(p.table, (p.D + BN - 1) / BN, G::MAX_ROWS);
   const int wn = (threadIdx.x >> 6) & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
-  Lin2Prog prog{p, p.H / kBK, wn, RowStager<2>(dyn_lds() + Ring::STAGES * Ring::STAGE)};
-  run_row_tiles<Lin2Prog::FM, FN>(prog, sched, ring, n_org);
+  Prog prog{p, p.H / kBK, wn};
+  run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);
+}
+
+__global__ __launch_bounds__(kThreads, 2) void lin2_scale_kernel(Lin2Args p) {
+  const ClockTrace trace(p.clk);
+  if (TileSched::tile_rows_of(p.table) > StdTiles::MAX_ROWS) lin2_scale_tiles<TallTiles>(p);
+  else lin2_scale_tiles<StdTiles>(p);
   trace.finish();
 }
+constexpr size_t kLin2Lds = std::max(Lin2Prog<TallTiles>::kLds, Lin2Prog<StdTiles>::kLds);
 
 // out[m] = sum_k rows[inv[m,k]]: one workgroup per token, 16-byte loads, fp32 accumulate.
 // The row numbers and then the rows are fetched 8 at a time with unconditional loads (a missing
@@ -407,8 +428,8 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
              nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<false>, Lin1Prog<false>::kLds, once);
-  lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, Lin1Prog<false>::kLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel<false>, kLin1FwdLds, once);
+  lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kLin1FwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -433,8 +454,8 @@ extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
              row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
              (bf16*)gz_blocked, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<true>, Lin1Prog<true>::kLds, once);
-  lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, Lin1Prog<true>::kLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin1_swiglu_kernel<true>, kLin1BwdLds, once);
+  lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kLin1BwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 
@@ -452,8 +473,8 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_blocked, const void* Wl2_NHD, 
   Lin2Args a{(const bf16*)h_blocked, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, Msum, clock_trace_buffer()};
   static std::once_flag once;
-  allow_lds(lin2_scale_kernel, Lin2Prog::kLds, once);
-  lin2_scale_kernel<<<persistent_grid(), kThreads, Lin2Prog::kLds, (hipStream_t)stream>>>(a);
+  allow_lds(lin2_scale_kernel, kLin2Lds, once);
+  lin2_scale_kernel<<<persistent_grid(), kThreads, kLin2Lds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
 

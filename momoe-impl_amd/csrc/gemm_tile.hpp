@@ -392,6 +392,10 @@ struct StageRing {
     return addr + slot(kt + head) * (STAGE * 2);
   }
   __device__ __forceinline__ void advance(int ktiles) { head = slot(head + ktiles); }
+  // After a tile's main loop (the ring has advanced): the one buffer that the next tile's first
+  // stages do not use, i.e. the finished tile's last stage.  Free for the epilogue once every
+  // wave has left the main loop (a barrier), until the next main loop's first barrier.
+  __device__ __forceinline__ bf16* free_buf() const { return lds + slot(head + FIRST) * STAGE; }
 };
 
 template <class AOp, class BOp, int NS>
@@ -551,11 +555,15 @@ struct RowTileGeometry {
   static constexpr int AROWS = (MAX_ROWS + 127) / 128 * 128;
   static constexpr int STAGES = NS_;
 };
-// 256-row tiles with a 4-stage ring: the kernel whose epilogue leaves no registers for more
+// 256-row tiles: the recomputing GEMM, whose epilogue leaves no registers for more, and any
+// launch whose tile table holds no taller tile (a routing in which no expert has more than 256
+// rows gains nothing from tall tiles and pays for their third deposit per stage and their
+// register pressure: a 16-token decode call ran 10% slower on them)
 using StdTiles = RowTileGeometry<4, 4>;
-// 320-row tiles: 10 accumulator fragments per wave, a 384-row stage buffer whose last 64 rows
-// repeat the tile's last row, and a 3-stage ring to pay for it in LDS
-using TallTiles = RowTileGeometry<5, 3>;
+// 320-row tiles: 10 accumulator fragments per wave and a 384-row stage buffer whose last 64 rows
+// repeat the tile's last row; four such stages are all of the CU's LDS (the epilogues stage
+// their stores in the ring's idle buffer)
+using TallTiles = RowTileGeometry<5, 4>;
 static_assert(TallTiles::MAX_ROWS == MOMOE_TILE_ROWS && StdTiles::MAX_ROWS == MOMOE_RECOMPUTE_TILE_ROWS,
               "tile heights promised by the header");
 
@@ -626,6 +634,10 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
   *(bf16x4*)p = pack_bf16x4(a, b, c, d);
 }
 
+// LDS the epilogues stage their stores in (RowStager below): 4 KiB per wave
+constexpr int kStageBytesPerWave = 32 * 64 * 2;                  // NF = 2
+constexpr size_t kEpilogueLds = (size_t)kWaves * kStageBytesPerWave;
+
 // ---- persistent tile loop ------------------------------------------------------------------------
 // Drives a workgroup through its (row tile, column block) pairs with everything a tile needs
 // from memory requested one tile ahead.  The tile program P supplies
@@ -634,7 +646,8 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
 //   late(tile, prep)                          loads that depend on gather()'s results: issued
 //                                             a tile later, under the tile's own main loop
 //   setup(tile, prep, A, B)                   operand set-up (may use gather()'s results)
-//   epilogue(tile, acc, prep)                 may use late()'s results
+//   epilogue(tile, acc, prep, staging)        may use late()'s results; staging = kEpilogueLds
+//                                             bytes of LDS for the workgroup
 //   ktiles                                    stages per tile
 // While tile t is multiplied: the table entry of tile t+2 and the gathered values of tile t+1
 // are in flight; after its main loop the first stages of tile t+1 are requested, then the
@@ -642,6 +655,7 @@ __device__ __forceinline__ void store_bf16x4(bf16* p, float a, float b, float c,
 template <int FM, int FN, class P, class AOp, class BOp, int NS>
 __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp, NS>& ring,
                                               const int (&n_org)[FN]) {
+  static_assert(StageRing<AOp, BOp, NS>::STAGE * sizeof(bf16) >= kEpilogueLds, "a stage buffer holds the store staging");
   TileCoord c0 = sched.next();
   if (!c0.valid) return;
   TileCoord c1 = sched.next();
@@ -668,7 +682,11 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
       prog.setup(c1, p1, A, B);
       gemm_issue_first(A, B, ring, prog.ktiles);  // travels during this tile's epilogue
     }
-    prog.epilogue(c0, acc, p0);
+    // the epilogue stages its stores in the ring's idle buffer: every wave must have read the
+    // last stage out of it
+    wait_lgkm0();
+    __builtin_amdgcn_s_barrier();
+    prog.epilogue(c0, acc, p0, ring.free_buf());
     if (!c1.valid) break;
     c0 = c1;
     p0 = p1;
@@ -682,8 +700,6 @@ __device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRi
 // requests.  Instead each wave passes one 32-row fragment row at a time through a private LDS
 // area (32 rows x 32*NF columns) and reads it back with 16 bytes per lane, lanes running along
 // the rows: stores then cover whole lines.  Wave-private: no barrier is involved.
-constexpr int kStageBytesPerWave = 32 * 64 * 2;                  // NF = 2
-constexpr size_t kEpilogueLds = (size_t)kWaves * kStageBytesPerWave;
 
 template <int NF>
 struct RowStager {

@@ -70,15 +70,35 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
   return v;
 }
 
+// Tile height for a routing (tile_rows = 0 asked for it).  A row tile streams its rows and a
+// 256-column block of the expert's weights, so a GEMM's time goes with the sum over the tiles of
+// (rows + 256): an expert of v rows costs v + 256 * (number of its tiles).  Tall tiles save whole
+// passes over the weights (an expert of 513..640 rows: two instead of three) but their kernels
+// are a few percent less efficient per tile: they are taken when they save more than 4 %.
+__device__ __forceinline__ int choose_tile_rows(const int32_t* sizes, int N, int lane) {
+  int64_t c_std = 0, c_tall = 0;
+  for (int i = lane; i < N; i += 64) {
+    const int v = sizes[i];
+    c_std += v + 256 * ((v + MOMOE_RECOMPUTE_TILE_ROWS - 1) / MOMOE_RECOMPUTE_TILE_ROWS);
+    c_tall += v + 256 * ((v + MOMOE_TILE_ROWS - 1) / MOMOE_TILE_ROWS);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    c_std += __shfl_xor(c_std, o);
+    c_tall += __shfl_xor(c_tall, o);
+  }
+  return c_tall * 26 < c_std * 25 ? MOMOE_TILE_ROWS : MOMOE_RECOMPUTE_TILE_ROWS;
+}
+
 __global__ __launch_bounds__(1024) void index_scan_kernel(
     int32_t* __restrict__ part, int N, int NC, int64_t msum_cap,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums,
-    int32_t* __restrict__ table, int tile_rows, int32_t* __restrict__ violations,
+    int32_t* __restrict__ table, int tile_rows_arg, int32_t* __restrict__ violations,
     int32_t* __restrict__ idx, int32_t* __restrict__ which) {
   __shared__ int32_t s_size[kMaxExperts];
   __shared__ int32_t s_cum[kMaxExperts];
   __shared__ int32_t s_first[kMaxExperts];
-  __shared__ int32_t s_total[2];
+  __shared__ int32_t s_total[3];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   // per expert: exclusive scan of the panel counts, in place
   for (int i = wave; i < N; i += 16) {
@@ -94,6 +114,7 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
   }
   __syncthreads();
   if (wave == 0) {
+    const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : choose_tile_rows(s_size, N, lane);
     int run_rows = 0, run_tiles = 0;
     for (int i0 = 0; i0 < N; i0 += 64) {
       const int i = i0 + lane;
@@ -116,6 +137,7 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
       if (overflow) atomicAdd(violations, 1);
       s_total[0] = overflow ? 0 : run_tiles;
       s_total[1] = run_rows;
+      s_total[2] = tile_rows;
       table[0] = overflow ? 0 : run_tiles;
       table[1] = tile_rows;
       table[2] = 0;
@@ -130,6 +152,7 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
     which[r] = 0;
   }
   if (s_total[0] == 0) return;
+  const int tile_rows = s_total[2];
   for (int i = t; i < N; i += 1024) {
     const int v = s_size[i];
     const int nt = (v + tile_rows - 1) / tile_rows;
@@ -204,7 +227,11 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
     int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
-    int tile_rows, int32_t* __restrict__ violations) {
+    int tile_rows_arg, int32_t* __restrict__ violations) {
+  // asked to choose the tile height: with at most 256 tokens no expert holds more than 256 rows,
+  // and taller tiles save nothing
+  const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
+  static_assert(kPanelTokens <= MOMOE_RECOMPUTE_TILE_ROWS, "one tile per expert in the one-launch kernel");
   __shared__ uint64_t ball[NGROUPS * kPanelExperts][4];  // tokens of expert i in wave w, as a lane mask
   __shared__ int32_t s_cum[NGROUPS * kPanelExperts];
   __shared__ int32_t s_wave[4][2];
@@ -348,8 +375,9 @@ extern "C" int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int6
 }
 
 extern "C" int64_t momoe_tile_table_ints(int64_t M, int64_t N, int64_t K, int tile_rows) {
-  if (M < 0 || N < 0 || K < 0 || tile_rows <= 0) return -1;
-  return kTileHeader + 4 * max_row_tiles(M * K, N, tile_rows);
+  if (M < 0 || N < 0 || K < 0 || tile_rows < 0) return -1;
+  // 0 = the library chooses between two heights: room for the shorter one
+  return kTileHeader + 4 * max_row_tiles(M * K, N, tile_rows > 0 ? tile_rows : MOMOE_RECOMPUTE_TILE_ROWS);
 }
 
 extern "C" int64_t momoe_index_workspace_bytes(int64_t M, int64_t N) {
@@ -367,7 +395,7 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
   if (!mask_NM || !sizes_N || !cumsums_N1 || !idx_Msum || !which_Msum || !inv_MK || !tile_table ||
       !workspace || !violations)
     return MOMOE_ERR_BAD_ARG;
-  if (M <= 0 || N <= 0 || K <= 0 || tile_rows <= 0) return MOMOE_ERR_BAD_ARG;
+  if (M <= 0 || N <= 0 || K <= 0 || tile_rows < 0) return MOMOE_ERR_BAD_ARG;
   if (N > kMaxExperts || M * K >= (1ll << 31) || M >= (1ll << 30)) return MOMOE_ERR_UNSUPPORTED;
   if (workspace_bytes < momoe_index_workspace_bytes(M, N)) return MOMOE_ERR_BAD_ARG;
   const int NC = (int)cdiv64(M, kPanelTokens), NG = (int)cdiv64(N, kPanelExperts);

@@ -21,7 +21,7 @@ namespace {
 
 constexpr int BX = 256;  // output rows per tile (features of A)
 constexpr int BY = 256;  // output columns per tile (features of B)
-constexpr int kStages = 3;  // ring depth: 16 stages per tile and L2-resident operands do not need more
+constexpr int kStages = 4;  // ring depth
 constexpr int kRingBytes = kStages * 2 * TLayout::LDS_ELEMS * 2;  // every operand kind: 16 KiB per stage
 constexpr size_t kWgradLds = kRingBytes + kEpilogueLds;  // stage ring + per-wave store staging
 constexpr int kMaxWgradExperts = 4096;  // 20 bytes of prefix sums per expert fit the stage ring

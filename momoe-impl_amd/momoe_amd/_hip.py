@@ -13,8 +13,9 @@ import torch  # noqa: F401  (loads the HIP runtime)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmomoe_hip.so")
 
-TILE_ROWS = 320            # MOMOE_TILE_ROWS: tile height of the table index_build returns
+TILE_ROWS = 320            # MOMOE_TILE_ROWS: the tallest row tile
 RECOMPUTE_TILE_ROWS = 256  # MOMOE_RECOMPUTE_TILE_ROWS: what lin1_swiglu_bwd takes
+AUTO_TILE_ROWS = 0         # index_build: the library picks one of the two from the routing
 GS_BLOCK = 128
 
 if not os.path.exists(LIB_PATH):
@@ -147,7 +148,7 @@ def abi_version():
 
 
 # ---------------------------------------------------------------- index build
-def index_build(mask_NM, K, static_scratch=False):
+def index_build(mask_NM, K, static_scratch=False, tile_rows=AUTO_TILE_ROWS):
     """mask_NM int32 [N,M] (any strides) -> dict of device tensors.
     See momoe_index_build in include/momoe_hip.h.  static_scratch=True goes through
     momoe_index_build_static: no workspace is allocated, the library's fixed array is used."""
@@ -161,18 +162,18 @@ def index_build(mask_NM, K, static_scratch=False):
     idx = torch.empty(msum, dtype=torch.int32, device=dev)
     which = torch.empty(msum, dtype=torch.int32, device=dev)
     inv = torch.empty(msum, dtype=torch.int32, device=dev)
-    table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, TILE_ROWS), dtype=torch.int32, device=dev)
+    table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, tile_rows), dtype=torch.int32, device=dev)
     violations = torch.zeros(1, dtype=torch.int32, device=dev)
     if static_scratch:
         _call("momoe_index_build_static", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N,
               K, _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv), _ptr(table),
-              TILE_ROWS, _ptr(violations), _stream())
+              tile_rows, _ptr(violations), _stream())
     else:
         ws_bytes = _lib.momoe_index_workspace_bytes(M, N)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         _call("momoe_index_build", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N, K,
               _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv), _ptr(table),
-              TILE_ROWS, _ptr(ws), ws_bytes, _ptr(violations), _stream())
+              tile_rows, _ptr(ws), ws_bytes, _ptr(violations), _stream())
     return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
             "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
 

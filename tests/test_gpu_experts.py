@@ -290,7 +290,7 @@ def test_recomputing_gemm_ignores_a_table_of_taller_tiles():
     M, D, H, N, K = 2048, 128, 64, 2, 1
     x, W1, _, mask, s, _ = make_layer_inputs(M, D, H, N, K, seed=5)
     dev = "cuda:0"
-    ib = _hip.index_build(mask.to(dev), K)
+    ib = _hip.index_build(mask.to(dev), K, tile_rows=_hip.TILE_ROWS)
     msum = M * K
     assert _hip.TILE_ROWS > _hip.RECOMPUTE_TILE_ROWS and int(ib["sizes_N"].max()) > _hip.RECOMPUTE_TILE_ROWS
     u = torch.randn(msum, H, device=dev).to(torch.bfloat16)

@@ -37,7 +37,12 @@ def _compare(mask, K, out):
         assert np.array_equal(out[k].numpy(), o[k]), k
     assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
     assert out["violations"].item() == 0
-    _check_table(out["tile_table"].numpy(), o, _hip.TILE_ROWS)
+    # left to choose, the library takes the taller tiles when they save more than 4 % of
+    # sum over the tiles of (rows + 256), the bytes a tile streams per k
+    def cost(rows):
+        return sum(int(v) + 256 * -(-int(v) // rows) for v in o["sizes_N"])
+    tall = cost(_hip.TILE_ROWS) * 26 < cost(_hip.RECOMPUTE_TILE_ROWS) * 25
+    _check_table(out["tile_table"].numpy(), o, _hip.TILE_ROWS if tall else _hip.RECOMPUTE_TILE_ROWS)
     # the table for another tile height, made from the prefix sums alone
     M = mask.shape[1]
     for rows in (_hip.RECOMPUTE_TILE_ROWS, _hip.TILE_ROWS, 32):
@@ -54,6 +59,7 @@ def _compare(mask, K, out):
     (16, 128, 8, 0, None),      # decode-sized
     (1, 4, 4, 0, None),
     (65536, 64, 8, 0, None),    # largest token count of the configurations
+    (4096, 64, 4, 0, None),     # experts of about 256 rows: half of them need a second 256-row tile
     # one token panel (M <= 256)
     (256, 128, 8, 0, None),     # a full panel
     (200, 300, 7, 2, None),     # 19 expert groups, two shared experts
@@ -64,6 +70,16 @@ def _compare(mask, K, out):
 def test_index_bit_exact(M, N, K, Ks, skew):
     mask, _ = make_routing(M, N, K, Ks, seed=11, skew=skew)
     _compare(mask, K, _run(mask, K))
+
+
+def test_index_with_a_given_tile_height():
+    from momoe_amd import _hip
+    mask, _ = make_routing(8192, 128, 8, seed=11)
+    o = oracle.index_build(mask)
+    for rows in (_hip.TILE_ROWS, _hip.RECOMPUTE_TILE_ROWS, 64):
+        out = _hip.index_build(mask.to("cuda:0"), 8, tile_rows=rows)
+        torch.cuda.synchronize()
+        _check_table(out["tile_table"].cpu().numpy(), o, rows)
 
 
 def test_index_strided_mask():

@@ -49,7 +49,7 @@ def test_static_scratch_allocates_nothing_and_refuses_oversized_inputs():
     rc = _hip._lib.momoe_index_build_static(
         d.data_ptr(), d.stride(0), d.stride(1), M, N, K, out["sizes_N"].data_ptr(),
         out["cumsums_N"].data_ptr(), out["idx_Msum"].data_ptr(), out["which_Msum"].data_ptr(),
-        out["inv_MK"].data_ptr(), out["tile_table"].data_ptr(), _hip.TILE_ROWS,
+        out["inv_MK"].data_ptr(), out["tile_table"].data_ptr(), _hip.AUTO_TILE_ROWS,
         out["violations"].data_ptr(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     free_after, _ = torch.cuda.mem_get_info()
