@@ -24,6 +24,11 @@ from . import _hip
 # every forward (one device synchronisation per call) and raise on a violation.
 CHECK_ROUTING = False
 
+# Row-tile height of the grouped GEMMs: _hip.AUTO_TILE_ROWS leaves the choice between 256 and 320
+# rows to the index build, which makes it on the device from the routing.  A fixed height (any
+# value up to _hip.TILE_ROWS) is for experiments and for tests that must cover both code paths.
+TILE_ROWS = _hip.AUTO_TILE_ROWS
+
 
 def _saved_rows(msum, save_percent):
     # momoe/momoe.py:251
@@ -66,7 +71,7 @@ class MoEFunction(torch.autograd.Function):
             mask = mask_NM.to(device=dev, dtype=torch.int32)
             s = s_NM.to(device=dev, dtype=torch.float32)
 
-            ib = _hip.index_build(mask, K)
+            ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS)
             idx, table = ib["idx_Msum"], ib["tile_table"]
             msum = M * K
             # nothing is kept for a backward that cannot happen (no input wants a gradient)

@@ -308,3 +308,27 @@ def test_recomputing_gemm_ignores_a_table_of_taller_tiles():
         assert bool((t == 7.0).all())
     own = _hip.tile_table_build(ib["cumsums_N"], M, K, _hip.RECOMPUTE_TILE_ROWS)
     assert not bool((run(own)[0] == 7.0).all())
+
+
+@pytest.mark.parametrize("sp", [0, 40])
+def test_both_row_tile_geometries_give_the_same_layer(sp):
+    """Experts of 1..700 rows on 256-row and on 320-row tiles (and on the library's own choice): the
+    contraction order does not depend on the tile height, so every result is bit-identical, and
+    the 320-row path is checked against the oracle like any other."""
+    from momoe_amd import _hip, experts
+    M, D, H, N, K = 1500, 160, 96, 12, 3
+    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, seed=21, skew=1.2)
+    assert int(mask.sum(1).max()) > 2 * _hip.RECOMPUTE_TILE_ROWS  # several tiles, ragged
+    outs = {}
+    try:
+        for rows in (_hip.RECOMPUTE_TILE_ROWS, _hip.TILE_ROWS, _hip.AUTO_TILE_ROWS, 288):
+            experts.TILE_ROWS = rows
+            outs[rows] = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
+    finally:
+        experts.TILE_ROWS = _hip.AUTO_TILE_ROWS
+    ref = run_oracle_layer(x, W1, W2, mask, s, dy)
+    _check_all(outs[_hip.TILE_ROWS], ref)
+    base = outs[_hip.RECOMPUTE_TILE_ROWS]
+    for rows, got in outs.items():
+        for k in base:
+            assert torch.equal(got[k], base[k]), (rows, k)
