@@ -30,13 +30,13 @@ PEAK_HBM_GBS = 8000.0
 # for a kernel that has not been measured.
 TRAFFIC_SOURCE = "profiles/momoe_layer_headline_fetch_size.txt + _write_size.txt"
 MEASURED_TRAFFIC_BYTES = {
-    "momoe_lin1_swiglu_fwd": 2 * 808836 * 1024 + 137116 * 1024,
-    "momoe_lin2_scale_fwd": 2 * 398250 * 1024 + 262144 * 1024,
-    "momoe_dgrad_h": 2 * 458030 * 1024 + 131072 * 1024,
-    "momoe_lin1_swiglu_bwd": 2 * 919950 * 1024 + 402739 * 1024,
-    "momoe_wgrad[Wl2]": 2 * 239251 * 1024 + 524372 * 1024,
-    "momoe_wgrad[Wl1]": 2 * 294344 * 1024 + 1048628 * 1024,
-    "momoe_dgrad_x": 2 * 795830 * 1024 + 262144 * 1024,
+    "momoe_lin1_swiglu_fwd": 2 * 708812 * 1024 + 148256 * 1024,
+    "momoe_lin2_scale_fwd": 2 * 425536 * 1024 + 271259 * 1024,
+    "momoe_dgrad_h": 2 * 388726 * 1024 + 131943 * 1024,
+    "momoe_lin1_swiglu_bwd": 2 * 915365 * 1024 + 402186 * 1024,
+    "momoe_wgrad[Wl2]": 2 * 238101 * 1024 + 524315 * 1024,
+    "momoe_wgrad[Wl1]": 2 * 295637 * 1024 + 1048598 * 1024,
+    "momoe_dgrad_x": 2 * 710413 * 1024 + 262144 * 1024,
 }
 
 
@@ -68,6 +68,8 @@ def kernel_bytes(M, D, H, N, K):
     return {
         # mask once, idx + inv (the reference's idx + which), cumsums, sizes
         "momoe_index_build": N * M * 4 + 2 * msum * 4 + (N + 1) * 4 + N * 8,
+        # prefix sums in, one 16-byte entry per 256-row tile out (launch-bound: a few microseconds)
+        "momoe_tile_table_build": (N + 1) * 4 + 16 * (msum // 256 + N),
         "momoe_combine": msum * D * 2 + M * D * 2 + msum * 4,
         "momoe_gs_scatter": msum * ((H + 127) // 128) * 4 + msum * 4 + msum * 4,
         # bf16 logits in; mask, s, p_sel out (4 bytes each); Ng, Ks per token
