@@ -368,10 +368,9 @@ struct TGatherDmaT {
 // ---- the k-loop -----------------------------------------------------------------------------
 // Ring of NS LDS stage buffers; `head` is the buffer of stage 0 of the current tile and is
 // carried from tile to tile by a persistent workgroup.  FIRST = NS - 1 stages of a tile are
-// requested ahead of its main loop (during the previous tile's epilogue).  Four buffers where the
-// weights stream k-row by k-row from HBM (three stages in flight cover that latency); three are
-// enough, and leave room for taller row tiles, where every line is fetched in two halves one
-// stage apart or is re-read from L2.
+// requested ahead of its main loop (during the previous tile's epilogue).  Every kernel here uses
+// four buffers: with three, the GEMMs whose weights stream k-row by k-row from HBM ran 3-7 % slower
+// (two stages in flight do not cover that latency); the others did not care.
 template <class AOp, class BOp, int NS>
 struct StageRing {
   static_assert(NS >= 3 && NS <= 5, "ring depth");
