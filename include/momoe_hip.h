@@ -74,6 +74,9 @@ int momoe_set_clock_trace(unsigned long long* ticks2);
  * int32[M*K] (sorted row of token m's k-th pair); tile_table
  * int32[momoe_tile_table_ints()] (device-side list of (expert,row-block) tiles
  * so that no GEMM launch depends on host knowledge of the routing);
+ * tile_rows: rows per row tile the table is built for, 1..MOMOE_TILE_ROWS, or 0: the library
+ * picks MOMOE_RECOMPUTE_TILE_ROWS or MOMOE_TILE_ROWS on the device (table[1] holds the choice);
+ * momoe_tile_table_ints(M, N, K, 0) sizes the table for either.
  * violations int32[1] += number of tokens whose pair count differs from K
  * (caller zeroes it; if the total pair count exceeds M*K the tile table is
  * emptied so later kernels touch nothing).
