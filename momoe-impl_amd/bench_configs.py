@@ -155,7 +155,7 @@ CHART_GRID = [
 
 
 if __name__ == "__main__":
-    assert torch.cuda.is_available() and _hip.abi_version() == 1
+    assert torch.cuda.is_available() and _hip.abi_version() == 2
     if "--chart" in sys.argv[1:]:
         for row in CHART_GRID:
             chart_row(*row)
