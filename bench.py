@@ -209,6 +209,20 @@ def main():
         ms_sustained = timed(layer, step, n_sus, 0)
     clock_sustained = ct.mhz()
 
+    # the same step captured once in a HIP graph and replayed (launch gaps only; the routing may
+    # change between replays: no launch is sized from it on the host)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(layer)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(layer)
+    ms_graph = timed(layer, lambda _l: graph.replay(), args.steps, args.warmup)
+    del graph
+
     # the other save setting
     other_sp = 100 if args.save_percent == 0 else 0
     layer2 = make_layer(other_sp)
@@ -277,6 +291,7 @@ def main():
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": M / (ms_fwd * 1e-3),
         "fwd_tflops": 6.0 * D * H * msum / ms_fwd / 1e9,
         f"ms_per_step_save_percent_{other_sp}": ms_other,
+        "graph_replay_ms_per_step": ms_graph,
         "sustained_ms_per_step": ms_sustained, "sustained_steps": n_sus,
         "sustained_tokens_per_s": M / (ms_sustained * 1e-3),
         "shader_clock_mhz": clock_timed, "sustained_shader_clock_mhz": clock_sustained,
