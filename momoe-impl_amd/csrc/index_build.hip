@@ -369,7 +369,7 @@ using namespace momoe;
 extern "C" int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int64_t Msum,
                                       int tile_rows, int32_t* tile_table, void* stream) {
   if (!cumsums_N1 || !tile_table || N <= 0 || Msum <= 0 || tile_rows <= 0) return MOMOE_ERR_BAD_ARG;
-  if (N > kMaxExperts || Msum >= (1ll << 31)) return MOMOE_ERR_UNSUPPORTED;
+  if (N > kMaxExperts || Msum >= (1ll << 31) || tile_rows > MOMOE_TILE_ROWS) return MOMOE_ERR_UNSUPPORTED;
   tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(cumsums_N1, (int)N, Msum, tile_rows, tile_table);
   return launch_status();
 }
@@ -397,6 +397,7 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
     return MOMOE_ERR_BAD_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || tile_rows < 0) return MOMOE_ERR_BAD_ARG;
   if (N > kMaxExperts || M * K >= (1ll << 31) || M >= (1ll << 30)) return MOMOE_ERR_UNSUPPORTED;
+  if (tile_rows > MOMOE_TILE_ROWS) return MOMOE_ERR_UNSUPPORTED;  // no GEMM takes taller tiles
   if (workspace_bytes < momoe_index_workspace_bytes(M, N)) return MOMOE_ERR_BAD_ARG;
   const int NC = (int)cdiv64(M, kPanelTokens), NG = (int)cdiv64(N, kPanelExperts);
   if (NG > 65535) return MOMOE_ERR_UNSUPPORTED;

@@ -82,6 +82,16 @@ def test_index_with_a_given_tile_height():
         _check_table(out["tile_table"].cpu().numpy(), o, rows)
 
 
+def test_tile_heights_no_kernel_takes_are_refused():
+    from momoe_amd import _hip
+    mask, _ = make_routing(300, 8, 2, seed=1)
+    with pytest.raises(RuntimeError):
+        _hip.index_build(mask.to("cuda:0"), 2, tile_rows=_hip.TILE_ROWS + 32)
+    ib = _hip.index_build(mask.to("cuda:0"), 2)
+    with pytest.raises(RuntimeError):
+        _hip.tile_table_build(ib["cumsums_N"], 300, 2, _hip.TILE_ROWS + 1)
+
+
 def test_index_strided_mask():
     mask, _ = make_routing(777, 24, 3, seed=2)
     strided = mask.T.contiguous().to("cuda:0").T  # strides (1, N)
