@@ -69,6 +69,16 @@ def test_random_small_shapes(seed):
     dev = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
     ref = run_oracle_layer(x, W1, W2, mask, s, dy)
     _check_all(dev, ref)
+    # the same through the 320-row code path of the forward and data-gradient GEMMs, which small
+    # routings never choose by themselves: bit-identical to the run above
+    from momoe_amd import _hip, experts
+    try:
+        experts.TILE_ROWS = _hip.TILE_ROWS
+        tall = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
+    finally:
+        experts.TILE_ROWS = _hip.AUTO_TILE_ROWS
+    for k in dev:
+        assert torch.equal(tall[k], dev[k]), k
 
 
 @pytest.mark.parametrize("gather_a", [True, False])
