@@ -23,21 +23,56 @@ for _p in (ROOT, os.path.join(ROOT, "momoe-impl_amd"), os.path.join(ROOT, "tests
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command
-# (profiles/momoe_layer_headline_{fetch,write}_size.txt; fetch scaled x2.0, write x1.0 by the
-# 256 MiB copy in the same runs).  Counters cannot be read from inside this process, so these are
-# the figures of the profile run named in TRAFFIC_SOURCE, not of the run that prints them; None
-# for a kernel that has not been measured.
-TRAFFIC_SOURCE = "profiles/momoe_layer_headline_fetch_size.txt + _write_size.txt"
-MEASURED_TRAFFIC_BYTES = {
-    "momoe_lin1_swiglu_fwd": 2 * 708812 * 1024 + 148256 * 1024,
-    "momoe_lin2_scale_fwd": 2 * 425536 * 1024 + 271259 * 1024,
-    "momoe_dgrad_h": 2 * 388726 * 1024 + 131943 * 1024,
-    "momoe_lin1_swiglu_bwd": 2 * 915365 * 1024 + 402186 * 1024,
-    "momoe_wgrad[Wl2]": 2 * 238101 * 1024 + 524315 * 1024,
-    "momoe_wgrad[Wl1]": 2 * 295637 * 1024 + 1048598 * 1024,
-    "momoe_dgrad_x": 2 * 710413 * 1024 + 262144 * 1024,
+# HBM bytes per launch come from two rocprofv3 --pmc runs of this same command (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), whose summaries are kept as text under profiles/ together with
+# the factor that the 256 MiB copy of --calibrate-copy gives each counter ("== scale:" line).
+# Counters cannot be read from inside this process, so the figures are those of the profiled run,
+# not of the run that prints them: they are parsed from the summaries every time, never typed in.
+TRAFFIC_FILES = {"fetch": "profiles/momoe_layer_headline_fetch_size.txt",
+                 "write": "profiles/momoe_layer_headline_write_size.txt"}
+TRAFFIC_SOURCE = " + ".join(TRAFFIC_FILES.values())
+# kernel names in the summaries -> entry points as this file names them
+PROFILE_KERNELS = {
+    "lin1_swiglu_kernel[fwd]": "momoe_lin1_swiglu_fwd", "lin1_swiglu_kernel[bwd]": "momoe_lin1_swiglu_bwd",
+    "lin2_scale_kernel": "momoe_lin2_scale_fwd", "dgrad_h_kernel": "momoe_dgrad_h",
+    "dgrad_x_kernel": "momoe_dgrad_x", "wgrad_kernel[Wl1": "momoe_wgrad[Wl1]",
+    "wgrad_kernel[Wl2": "momoe_wgrad[Wl2]", "combine_kernel": "momoe_combine",
 }
+
+
+def parse_counter_summary(path, counter):
+    """(scale, {kernel name in the summary: average counter value per dispatch})."""
+    scale, rows = None, {}
+    with open(path) as f:
+        for line in f:
+            if line.startswith("== scale:"):
+                scale = float(line.split(":", 1)[1].split()[0])
+            elif f" {counter} " in line and not line.startswith(("#", "==")):
+                name, rest = line.split(f" {counter} ", 1)
+                rows[name.strip()] = float(rest.split()[0])
+    if scale is None:
+        raise ValueError(f"{path}: no '== scale:' line")
+    return scale, rows
+
+
+def measured_traffic(root=ROOT):
+    """{entry point: HBM bytes per launch = scale_f * FETCH_SIZE + scale_w * WRITE_SIZE} from the
+    committed counter summaries; empty when they are not there."""
+    try:
+        sf, fetch = parse_counter_summary(os.path.join(root, TRAFFIC_FILES["fetch"]), "FETCH_SIZE")
+        sw, write = parse_counter_summary(os.path.join(root, TRAFFIC_FILES["write"]), "WRITE_SIZE")
+    except (OSError, ValueError):
+        return {}
+    out = {}
+    for prof_name, entry in PROFILE_KERNELS.items():
+        f = [v for k, v in fetch.items() if k.startswith(prof_name)]
+        w = [v for k, v in write.items() if k.startswith(prof_name)]
+        if len(f) == 1 and len(w) == 1:
+            out[entry] = int(round((sf * f[0] + sw * w[0]) * 1024))
+    return out
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic()
 
 
 def headline_inputs(M, D, H, N, K, seed=0):
@@ -62,6 +97,23 @@ def kernel_flops(D, H, msum):
     }
 
 
+def gemm_algorithmic_bytes(M, D, H, N, K):
+    """Bytes a GEMM launch must move at least: every input read once, every output written once
+    (weights 2 bytes per element; x and G_y are read once although gathered)."""
+    msum = M * K
+    w1, w2 = N * D * 2 * H * 2, N * H * D * 2
+    xb, hb, ysb, gzb = M * D * 2, msum * H * 2, msum * D * 2, msum * 2 * H * 2
+    return {
+        "momoe_lin1_swiglu_fwd": w1 + xb + hb,
+        "momoe_lin2_scale_fwd": w2 + hb + ysb,
+        "momoe_dgrad_h": w2 + xb + hb,
+        "momoe_lin1_swiglu_bwd": w1 + xb + hb + gzb + hb + msum * 4 * ((H + 127) // 128),
+        "momoe_wgrad[Wl2]": hb + xb + w2,
+        "momoe_wgrad[Wl1]": xb + gzb + w1,
+        "momoe_dgrad_x": w1 + gzb + ysb,
+    }
+
+
 def kernel_bytes(M, D, H, N, K):
     """Algorithmic HBM bytes per launch of the bandwidth-bound kernels."""
     msum = M * K
@@ -81,37 +133,127 @@ def kernel_bytes(M, D, H, N, K):
     }
 
 
-def cpu_baseline(D, H, N, K, budget_s=25.0):
-    """The oracle MoE layer as `MoE.forward` runs it (router -> per-expert loop -> bias update,
-    momoe/sample_moe.py:59-68) plus its autograd backward, in fp32 on the host cores, on a
-    reduced token count of the same layer."""
+def _host_cpus():
+    """(logical CPUs the OS shows, physical cores, CPUs this process may run on)."""
+    logical = os.cpu_count() or 1
+    try:
+        import psutil
+        physical = psutil.cpu_count(logical=False) or logical
+    except Exception:
+        physical = logical
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except Exception:
+        usable = logical
+    return logical, physical, usable
+
+
+def _oracle_moe_pass(oracle, torch, x, Wg, W1, W2, biases, dy, K, dtype, backward):
+    """One pass of the oracle MoE layer as `MoE.forward` runs it (router -> experts -> bias
+    update, momoe/sample_moe.py:59-68) and, with `backward`, its backward (experts, then router:
+    momoe/momoe.py:881-903, momoe/topk_router.py:127-145), every product formed once."""
+    M, D = x.shape
+    N = W1.shape[0]
+    r = oracle.router_forward(x, Wg, biases, N, K, 0)
+    mask, s = r["mask_NM"], r["s_NM"]
+    if not backward:
+        y = oracle.experts_forward(x, W1, W2, mask, s, dtype=dtype)
+        oracle.bias_update(biases, (mask != 0).sum(1), M, K, 0, 1e-4)
+        return y
+    y, G_x, G_W1, G_W2, G_s = oracle.experts_forward_backward(x, W1, W2, mask, s, dy, dtype=dtype)
+    oracle.bias_update(biases, (mask != 0).sum(1), M, K, 0, 1e-4)
+    G_logit = oracle.router_backward_closed_form(G_s.float(), r["p_sel_MN"], s, r["Ng_M"], r["Ks_M"],
+                                                 mask, 0, round_bf16=True).to(dtype)
+    Wgd, xd = Wg.to(dtype), x.to(dtype)
+    G_x = G_x + G_logit @ Wgd.T
+    G_Wg = xd.T @ G_logit
+    return y, G_x, G_W1, G_W2, G_Wg
+
+
+def cpu_baseline(D, H, N, K, budget_s=28.0):
+    """The CPU restatement of `MoE.forward` (router -> per-expert loop -> bias update) and of its
+    backward, timed on the host cores: forward and forward+backward, fp32 and bf16, on the tiny
+    reference configuration and on a 1024-token slice of the headline layer.  `value` is the
+    fp32 forward+backward rate of the headline slice.  A plain torch.mm on the same threads is
+    timed beside it, so the figure can be read against what these cores give a GEMM."""
     import torch
     import oracle
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
-    Ms = 1024
-    x, W1, W2, _, _, dy = headline_inputs(Ms, D, H, N, K, seed=1)
-    Wg = torch.randn(D, N, generator=torch.Generator().manual_seed(2)) / D ** 0.5
-    moe = oracle.OracleMoE(D, H, N, K, 0, Wg_DN=Wg, Wl1_ND2H=W1.float(), Wl2_NHD=W2.float())
-    xf = x.bfloat16().float().reshape(1, Ms, D).requires_grad_()
-    dyf = dy.reshape(1, Ms, D)
-    times = []
-    t_start = time.time()
-    for it in range(4):
+    from helpers import make_layer_inputs
+    logical, physical, usable = _host_cpus()
+    # the threads torch starts with: OMP_NUM_THREADS where the machine sets it (a box shared
+    # between jobs says there how many cores are this job's), else every CPU of the process
+    threads = torch.get_num_threads()
+    t_begin = time.time()
+
+    def best_of(fn, cap_s, min_runs=3, max_runs=5):
+        fn()  # warm-up (page faults, thread pool start)
+        times = []
         t0 = time.time()
-        y = moe(xf)
-        y.backward(dyf)
-        dt = time.time() - t0
-        moe.zero_grad(set_to_none=True)
-        xf.grad = None
-        if it > 0:
-            times.append(dt)
-        if time.time() - t_start > budget_s and times:
-            break
-    best = min(times)
-    return {"value": Ms / best, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"oracle MoE (router + experts + bias update) fwd+bwd, fp32, {Ms} of 8192 tokens of the "
-                      f"headline layer (D={D}, H={H}, N={N}, K={K}), best of {len(times)} runs, {best:.3f} s each"}
+        while len(times) < max_runs and (len(times) < min_runs or time.time() - t0 < cap_s):
+            t = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t)
+            if time.time() - t0 > 2.5 * cap_s:
+                break
+        return min(times), len(times)
+
+    def mm_rate(m, k, n, dtype):
+        a, b = torch.randn(m, k).to(dtype), torch.randn(k, n).to(dtype)
+        t, _ = best_of(lambda: torch.mm(a, b), 0.5, 3, 10)
+        return 2.0 * m * k * n / t / 1e9
+
+    results = {}
+    # C1: the reference's own CPU-sized case (B=2, S=64, D=128, H=64, N=8, K=2)
+    tiny = dict(M=128, D=128, H=64, N=8, K=2)
+    # the headline layer at 1024 of its 8192 tokens: every expert, 64 rows per expert on average
+    slice_ = dict(M=1024, D=D, H=H, N=N, K=K)
+    for label, c in (("tiny", tiny), ("headline_slice", slice_)):
+        x, W1, W2, _, _, dy = make_layer_inputs(c["M"], c["D"], c["H"], c["N"], c["K"], seed=1)
+        x = x.bfloat16().float()
+        Wg = (torch.randn(c["D"], c["N"], generator=torch.Generator().manual_seed(2)) / c["D"] ** 0.5).bfloat16()
+        biases = torch.zeros(c["N"])
+        unit = float(c["D"]) * c["H"] * c["M"] * c["K"]
+        for dtype, dname in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            W1d, W2d, xd, dyd = W1.to(dtype), W2.to(dtype), x.to(dtype), dy.to(dtype)
+            for backward in (False, True):
+                left = budget_s - (time.time() - t_begin)
+                cap = 0.2 if label == "tiny" else max(0.5, left / (5 if dtype == torch.float32 else 3))
+                with torch.no_grad():
+                    t, n = best_of(lambda: _oracle_moe_pass(oracle, torch, xd, Wg, W1d, W2d, biases, dyd,
+                                                            c["K"], dtype, backward), cap)
+                key = f"{label}_{dname}_{'fwd_bwd' if backward else 'fwd'}"
+                results[key] = {"tokens_per_s": c["M"] / t, "seconds": t, "runs": n,
+                                "gflops": (18.0 if backward else 6.0) * unit / t / 1e9}
+            del W1d, W2d
+    rows = slice_["M"] * K // N
+
+    def mm_rate_streaming(dtype):
+        # the up projection of the slice as the layer meets it: one [rows, D] x [D, 2H] product
+        # per expert, each with its own weights (N * D * 2H elements streamed from memory)
+        a, w = torch.randn(rows, D).to(dtype), W1.to(dtype)
+        t, _ = best_of(lambda: [torch.mm(a, w[i]) for i in range(N)], 0.5, 3, 5)
+        return 2.0 * rows * D * 2 * H * N / t / 1e9
+
+    results["torch_mm_gflops"] = {
+        f"fp32_[{rows},{D}]x[{D},{2 * H}]_one_weight_in_cache": mm_rate(rows, D, 2 * H, torch.float32),
+        f"fp32_[{rows},{D}]x[{D},{2 * H}]_per_expert_weights": mm_rate_streaming(torch.float32),
+        "fp32_[2048,2048]x[2048,2048]": mm_rate(2048, 2048, 2048, torch.float32),
+        f"bf16_[{rows},{D}]x[{D},{2 * H}]_per_expert_weights": mm_rate_streaming(torch.bfloat16),
+    }
+    head = results["headline_slice_fp32_fwd_bwd"]
+    return {"value": head["tokens_per_s"], "unit": "tokens/s", "cores": threads, "kind": "port",
+            "logical_cpus": logical, "physical_cores": physical, "usable_cpus": usable,
+            "torch_threads": threads,
+            "sample": f"CPU oracle of the MoE layer (router + experts + bias update; backward: experts then "
+                      f"router), every GEMM executed once (18*D*H flops per pair, no autograd), on "
+                      f"{threads} torch threads ({physical} physical / {logical} logical CPUs on the host, "
+                      f"{usable} usable by this process): value = fp32 forward+backward of {slice_['M']} of "
+                      f"the 8192 tokens of the headline layer (D={D}, H={H}, N={N}, K={K}; {rows} rows per "
+                      f"expert), best of {head['runs']} runs of {head['seconds']:.3f} s = "
+                      f"{head['gflops']:.0f} GFLOP/s; `variants` holds fp32 and bf16, forward and "
+                      f"forward+backward, for that slice and for the tiny reference configuration "
+                      f"(128 tokens, D=128, H=64, N=8, K=2), and torch.mm rates on the same threads",
+            "variants": results}
 
 
 def main():
@@ -272,11 +414,42 @@ def main():
             kernels[k]["frac_hbm_peak"] = kernels[k]["hbm_gbs"] / PEAK_HBM_GBS
     dom = max((k for k in kernels if k in flops),
               key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
+    alg_bytes = gemm_algorithmic_bytes(M, D, H, N, K)
+    for k, b in alg_bytes.items():
+        if k in kernels:
+            kernels[k]["algorithmic_bytes"] = b
+            if k in MEASURED_TRAFFIC_BYTES:
+                kernels[k]["traffic_bytes"] = MEASURED_TRAFFIC_BYTES[k]
+                kernels[k]["traffic_over_algorithmic"] = MEASURED_TRAFFIC_BYTES[k] / b
     roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": kernels[dom]["tflops"] / PEAK_BF16_TFLOPS,
                 "avg_launch_ms": kernels[dom]["avg_ms"], "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                "traffic_over_algorithmic": (MEASURED_TRAFFIC_BYTES[dom] / alg_bytes[dom]
+                                             if dom in MEASURED_TRAFFIC_BYTES else None),
                 "traffic_source": TRAFFIC_SOURCE if dom in MEASURED_TRAFFIC_BYTES else None,
                 "shader_clock_mhz": clock_timed}
+
+    # what this machine gives a plain GEMM of the up projection's size, outside the timed
+    # region: the vendor library on perfectly balanced experts (no gather, no epilogue, no ragged
+    # tiles), and the matrix pipe alone on register operands of the layer's kind of data
+    xa = torch.randn(N, msum // N, D, device=dev).to(torch.bfloat16)
+    for _ in range(3):
+        torch.bmm(xa, layer.Wl1_ND2H.data)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        torch.bmm(xa, layer.Wl1_ND2H.data)
+    e1.record()
+    torch.cuda.synchronize()
+    vendor_ms = e0.elapsed_time(e1) / 10
+    del xa
+    machine = {"vendor_gemm_ms": vendor_ms,
+               "vendor_gemm": f"torch.bmm {N} x [{msum // N},{D}] x [{D},{2 * H}] bf16 (the flops of momoe_lin1_swiglu_fwd)",
+               "vendor_gemm_tflops": 4.0 * D * H * msum / vendor_ms / 1e9}
+    for kind in ("gaussian", "zeros"):
+        tf, mhz = _hip.mfma_rate_probe(kind)
+        machine[f"mfma_only_tflops_{kind}"] = tf
+        machine[f"mfma_only_shader_clock_mhz_{kind}"] = mhz
 
     useful = 18.0 * D * H * msum
     out = {
@@ -297,7 +470,7 @@ def main():
         "shader_clock_mhz": clock_timed, "sustained_shader_clock_mhz": clock_sustained,
         "ms_per_step_with_router": ms_moe, "tokens_per_s_with_router": M / (ms_moe * 1e-3),
         "peak_activation_mib": peak_extra_mib,
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline, "machine": machine, "kernels": kernels,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(D, H, N, K)

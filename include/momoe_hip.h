@@ -63,6 +63,21 @@ const char* momoe_status_string(int status);
  */
 int momoe_set_clock_trace(unsigned long long* ticks2);
 
+/* Measurement aid, no counterpart in the reference: what the matrix pipe of this machine
+ * sustains on a given kind of operand data.  Launches one workgroup of 8 wavefronts per CU whose
+ * waves do nothing but issue the GEMMs' MFMA (v_mfma_f32_32x32x16_bf16, the 2 x 4 fragment tile
+ * of one wave) `iters` x 16 times on operands read once from operands_64KiB (4096 x 16 bytes of
+ * bf16 values: the row-side operand's fragments come from the first half, the column-side
+ * operand's from the second half).  The
+ * rate depends on the data: the chip is power-limited under sustained MFMA load.
+ * sink_512: 512 floats of scratch (not written in practice).  ticks2 (may be NULL): device
+ * pointer to two 64-bit counters that receive the shader-clock ticks and the 100 MHz ticks of
+ * one wavefront.  Returns the number of floating-point operations of the launch (time it with
+ * events on `stream`), or -1 on a bad argument / failed launch.
+ */
+int64_t momoe_mfma_rate_probe(const void* operands_64KiB, float* sink_512, int iters,
+                              unsigned long long* ticks2, void* stream);
+
 /* ---- routing index -------------------------------------------------------
  * Replaces find_used_experts + scatter_cols_kernel (momoe/momoe.py:821-842,
  * 760-815) and the torch.sum at :830.
@@ -74,7 +89,9 @@ int momoe_set_clock_trace(unsigned long long* ticks2);
  * int32[M*K] (sorted row of token m's k-th pair); tile_table
  * int32[momoe_tile_table_ints()] (device-side list of (expert,row-block) tiles
  * so that no GEMM launch depends on host knowledge of the routing);
- * tile_rows: rows per row tile the table is built for, 1..MOMOE_TILE_ROWS, or 0: the library
+ * tile_rows: rows per row tile the table is built for, a multiple of 32 from 32 to
+ * MOMOE_TILE_ROWS (anything else: MOMOE_ERR_UNSUPPORTED; the GEMMs deal whole 32-row fragment
+ * rows to an expert's tiles), or 0: the library
  * picks MOMOE_RECOMPUTE_TILE_ROWS or MOMOE_TILE_ROWS on the device (table[1] holds the choice);
  * momoe_tile_table_ints(M, N, K, 0) sizes the table for either.
  * violations int32[1] += number of tokens whose pair count differs from K
@@ -94,7 +111,8 @@ int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m
 /* A tile table for another tile height, from the prefix sums of a finished momoe_index_build
  * (no counterpart in the reference: its launchers size their grids on the host).  Msum = M*K, the
  * rows the sorted matrices were allocated for; tile_table int32[momoe_tile_table_ints(M, N, K,
- * tile_rows)].  Same contents as the table momoe_index_build writes for that tile_rows.
+ * tile_rows)].  Same contents as the table momoe_index_build writes for that tile_rows (a
+ * multiple of 32 from 32 to MOMOE_TILE_ROWS; 0 is not accepted here).
  */
 int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int64_t Msum, int tile_rows,
                            int32_t* tile_table, void* stream);

@@ -43,9 +43,11 @@ def routing(M, N, K, Ks, skew, gen):
 
 
 def balanced_routing(M, N, K, gen):
-    """Every expert gets exactly M*K/N tokens: token m goes to experts m + j*N/K (mod N)."""
-    assert N % K == 0
-    cols = (torch.arange(M, device=DEV)[:, None] + torch.arange(K, device=DEV)[None, :] * (N // K)) % N
+    """The M*K pairs dealt to the experts round-robin: pair j of token m goes to expert
+    (m*K + j) mod N, K consecutive (hence distinct) experts per token, and every expert gets
+    floor(M*K/N) or ceil(M*K/N) tokens whether or not K divides N."""
+    assert K <= N
+    cols = (torch.arange(M, device=DEV)[:, None] * K + torch.arange(K, device=DEV)[None, :]) % N
     chosen = torch.zeros(M, N, dtype=torch.bool, device=DEV).scatter_(1, cols, True)
     w = torch.rand(M, N, generator=gen, device=DEV) * chosen
     return chosen.T.to(torch.int32).contiguous(), (w / w.sum(-1, keepdim=True)).contiguous().T
@@ -148,7 +150,7 @@ def chart_row(B, S, D, H, N, K, kind, steps=5):
 
 CHART_GRID = [
     (2, 512, 1024, 512, 32, 4, "balanced"), (4, 2048, 2048, 1024, 64, 8, "balanced"),
-    (4, 2048, 2048, 1024, 64, 8, "skewed"), (6, 2048, 2048, 1280, 64, 6, "random"),
+    (4, 2048, 2048, 1024, 64, 8, "skewed"), (6, 2048, 2048, 1280, 64, 6, "balanced"),
     (4, 1920, 2176, 1152, 64, 6, "random"), (8, 4096, 2048, 1024, 128, 8, "balanced"),
     (8, 4096, 2048, 1024, 128, 8, "skewed"), (8, 8192, 2048, 1024, 128, 8, "balanced"),
 ]

@@ -269,7 +269,8 @@ __global__ __launch_bounds__(256) void gs_scatter_kernel(const float* __restrict
                                                          float* __restrict__ gs, int M, int N,
                                                          int64_t msum) {
   const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= msum || r >= cumsums[N]) return;
+  // more pairs than rows: the routing was refused (empty tile table), dL/ds stays zero
+  if (r >= msum || r >= cumsums[N] || cumsums[N] > msum) return;
   // expert of row r: the i with cumsums[i] <= r < cumsums[i+1]
   int lo = 0, hi = N;  // invariant: cumsums[lo] <= r < cumsums[hi]
   while (hi - lo > 1) {
@@ -306,8 +307,8 @@ extern "C" int momoe_dgrad_h(const void* Gy_MD, const void* Wl2_NHD, const int32
   if (st != MOMOE_OK) return st;
   DhArgs a{(const bf16*)Gy_MD, (const bf16*)Wl2_NHD, idx_Msum, tile_table, (bf16*)u_MsumH, (int)D,
            (int)H, clock_trace_buffer()};
-  static std::once_flag once;
-  allow_lds(dgrad_h_kernel, kDhLds, once);
+  static LdsLimit lds;
+  if (!allow_lds(dgrad_h_kernel, kDhLds, lds)) return MOMOE_ERR_LAUNCH;
   dgrad_h_kernel<<<persistent_grid(), kThreads, kDhLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
@@ -360,8 +361,8 @@ extern "C" int momoe_dgrad_x(const void* gz_blocked, const void* Wl1_ND2H,
   if (st != MOMOE_OK) return st;
   DxArgs a{(const bf16*)gz_blocked, (const bf16*)Wl1_ND2H, tile_table, (bf16*)gxs_MsumD, (int)D,
            (int)H, Msum, clock_trace_buffer()};
-  static std::once_flag once;
-  allow_lds(dgrad_x_kernel, kDxLds, once);
+  static LdsLimit lds;
+  if (!allow_lds(dgrad_x_kernel, kDxLds, lds)) return MOMOE_ERR_LAUNCH;
   dgrad_x_kernel<<<persistent_grid(), kThreads, kDxLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }

@@ -427,8 +427,8 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_blocked,
              (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
              nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, Msum, clock_trace_buffer()};
-  static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<false>, kLin1FwdLds, once);
+  static LdsLimit lds;
+  if (!allow_lds(lin1_swiglu_kernel<false>, kLin1FwdLds, lds)) return MOMOE_ERR_LAUNCH;
   lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kLin1FwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
@@ -453,8 +453,8 @@ extern "C" int momoe_lin1_swiglu_bwd(const void* x_MD, const void* Wl1_ND2H,
   Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, nullptr, nullptr,
              row_lo, Msum, (int)D, (int)H, (const bf16*)u_MsumH, s_NM, s_stride_n, s_stride_m,
              (bf16*)gz_blocked, (bf16*)hsT_GH32, ld_hsT, gs_part, Msum, clock_trace_buffer()};
-  static std::once_flag once;
-  allow_lds(lin1_swiglu_kernel<true>, kLin1BwdLds, once);
+  static LdsLimit lds;
+  if (!allow_lds(lin1_swiglu_kernel<true>, kLin1BwdLds, lds)) return MOMOE_ERR_LAUNCH;
   lin1_swiglu_kernel<true><<<persistent_grid(), kThreads, kLin1BwdLds, (hipStream_t)stream>>>(a);
   return launch_status();
 }
@@ -472,8 +472,8 @@ extern "C" int momoe_lin2_scale_fwd(const void* h_blocked, const void* Wl2_NHD, 
   if (st != MOMOE_OK) return st;
   Lin2Args a{(const bf16*)h_blocked, (const bf16*)Wl2_NHD, s_NM, s_stride_n, s_stride_m,
              idx_Msum, tile_table, (bf16*)ys_MsumD, (int)D, (int)H, Msum, clock_trace_buffer()};
-  static std::once_flag once;
-  allow_lds(lin2_scale_kernel, kLin2Lds, once);
+  static LdsLimit lds;
+  if (!allow_lds(lin2_scale_kernel, kLin2Lds, lds)) return MOMOE_ERR_LAUNCH;
   lin2_scale_kernel<<<persistent_grid(), kThreads, kLin2Lds, (hipStream_t)stream>>>(a);
   return launch_status();
 }

@@ -62,6 +62,7 @@
 // column 8*(r/4) + 4*(lane/32) + r%4.  Row-wise epilogues (per-row scale,
 // SwiGLU pairing, row reductions) are then lane-local and stores are 8-byte.
 #pragma once
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -592,22 +593,36 @@ __device__ __forceinline__ bf16* dyn_lds() {
   return momoe_lds;
 }
 
-// Kernels use more than the 64 KiB of LDS a launch gets by default: raise the limit once.
+// Kernels use more than the 64 KiB of LDS a launch gets by default: the limit is raised once per
+// kernel, and the outcome kept, so that an entry point whose kernel cannot have its LDS reports
+// it instead of failing at every launch for no visible reason.
+struct LdsLimit {
+  std::once_flag once;
+  bool ok = false;
+};
 template <class Kernel>
-inline void allow_lds(Kernel kernel, size_t bytes, std::once_flag& once) {
-  std::call_once(once, [&] {
-    (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)bytes);
+inline bool allow_lds(Kernel kernel, size_t bytes, LdsLimit& lim) {
+  std::call_once(lim.once, [&] {
+    lim.ok = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)bytes) == hipSuccess;
+    if (!lim.ok) (void)hipGetLastError();
   });
+  return lim.ok;
 }
 
 // number of persistent workgroups: one per CU of the current device, rounded to the 8 XCDs
+// (the CU count of a device is looked up once)
 inline int persistent_grid() {
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-      cus <= 0)
-    cus = 256;
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached[dev].store(cus, std::memory_order_relaxed);
+  }
   return (cus + 7) / 8 * 8;
 }
 

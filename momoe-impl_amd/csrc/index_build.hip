@@ -177,6 +177,7 @@ __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int m = c * kPanelTokens + t;
   const int64_t msum = (int64_t)M * K;
+  const bool overflow = (int64_t)cumsums[N] > msum;
   const uint32_t bits = load_panel_bits(mask, sn, sm, M, N, g, m);
   uint64_t ballots[kPanelExperts];
 #pragma unroll
@@ -201,8 +202,10 @@ __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
       if (row < msum) {
         idx[row] = m;
         which[row] = k;
-        if (k < K) inv[(int64_t)m * K + k] = (int32_t)row;
       }
+      // more pairs than rows: the GEMMs get an empty tile table and write nothing, so no token
+      // may point at a row (the combine then gives zeros instead of unwritten memory)
+      if (k < K) inv[(int64_t)m * K + k] = row < msum && !overflow ? (int32_t)row : -1;
       ++k;
     }
   }
@@ -307,8 +310,8 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
       if (row < msum) {
         idx[row] = t;
         which[row] = k;
-        if (k < K) inv[(int64_t)t * K + k] = (int32_t)row;
       }
+      if (k < K) inv[(int64_t)t * K + k] = row < msum && !overflow ? (int32_t)row : -1;
       ++k;
     }
   }
@@ -366,10 +369,18 @@ __global__ __launch_bounds__(1024) void tile_table_kernel(const int32_t* __restr
 
 using namespace momoe;
 
+// The GEMMs deal an expert's 32-row fragment rows to its ceil(rows / tile_rows) tiles: with a tile
+// height below 32, or one that is not a whole number of fragment rows, there would be more tiles
+// than fragment rows (tiles without rows, addressed past the expert's end) or tiles taller than
+// the height the table promises.  No GEMM takes tiles above MOMOE_TILE_ROWS.
+static bool tile_height_ok(int tile_rows) {
+  return tile_rows >= 32 && tile_rows <= MOMOE_TILE_ROWS && tile_rows % 32 == 0;
+}
+
 extern "C" int momoe_tile_table_build(const int32_t* cumsums_N1, int64_t N, int64_t Msum,
                                       int tile_rows, int32_t* tile_table, void* stream) {
   if (!cumsums_N1 || !tile_table || N <= 0 || Msum <= 0 || tile_rows <= 0) return MOMOE_ERR_BAD_ARG;
-  if (N > kMaxExperts || Msum >= (1ll << 31) || tile_rows > MOMOE_TILE_ROWS) return MOMOE_ERR_UNSUPPORTED;
+  if (N > kMaxExperts || Msum >= (1ll << 31) || !tile_height_ok(tile_rows)) return MOMOE_ERR_UNSUPPORTED;
   tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(cumsums_N1, (int)N, Msum, tile_rows, tile_table);
   return launch_status();
 }
@@ -397,7 +408,7 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
     return MOMOE_ERR_BAD_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || tile_rows < 0) return MOMOE_ERR_BAD_ARG;
   if (N > kMaxExperts || M * K >= (1ll << 31) || M >= (1ll << 30)) return MOMOE_ERR_UNSUPPORTED;
-  if (tile_rows > MOMOE_TILE_ROWS) return MOMOE_ERR_UNSUPPORTED;  // no GEMM takes taller tiles
+  if (tile_rows != 0 && !tile_height_ok(tile_rows)) return MOMOE_ERR_UNSUPPORTED;
   if (workspace_bytes < momoe_index_workspace_bytes(M, N)) return MOMOE_ERR_BAD_ARG;
   const int NC = (int)cdiv64(M, kPanelTokens), NG = (int)cdiv64(N, kPanelExperts);
   if (NG > 65535) return MOMOE_ERR_UNSUPPORTED;

@@ -304,8 +304,16 @@ __device__ __forceinline__ f32x4* partial_piece(float* ws, int slot, int i, int 
 // them up.
 // CUT = false is the launch in which no expert can reach the cutting length (the host knows:
 // an expert holds at most M rows): the bookkeeping of pieces is compiled out.
+// A routing with more pairs than sorted rows (cumsums[N] > Msum) got an empty tile table: the
+// GEMMs before this one wrote nothing, so no expert has rows to contract over and every weight
+// gradient is zero.  Row counts are clamped to p.msum everywhere: clamp them to nothing.
+__device__ __forceinline__ void drop_rows_of_an_overflowed_routing(WgradArgs& p) {
+  if (load_uniform(p.cumsums + p.N) > p.msum) p.msum = 0;
+}
+
 template <bool CUT, class AOp, class BOp, int FM, int FN>
 __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
+  drop_rows_of_an_overflowed_routing(p);
   using Ring = StageRing<AOp, BOp, kStages>;
   static_assert(Ring::BYTES == kRingBytes, "ring size assumed by the launch");
   const ClockTrace trace(p.clk);
@@ -449,6 +457,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_kernel(WgradArgs p) {
 // bf16 result; one workgroup per output tile, same register layout as the GEMM.
 template <int FM, int FN>
 __global__ __launch_bounds__(kThreads) void wgrad_reduce_kernel(WgradArgs p) {
+  drop_rows_of_an_overflowed_routing(p);
   const int tpe = p.tiles_x * p.tiles_y;
   const Plan pl = build_plan(p, tpe);
   const int ncut = pl.ctiles[p.N];
@@ -499,13 +508,14 @@ extern "C" int64_t momoe_wgrad_workspace_bytes(int64_t N, int64_t X, int64_t Y, 
 namespace {
 template <class AOp, class BOp, int FM, int FN>
 int launch_wgrad(const WgradArgs& a, bool can_cut, int grid, hipStream_t st) {
-  static std::once_flag once, once_cut, once_reduce;
+  static LdsLimit once, once_cut, once_reduce;
   if (!can_cut) {
-    allow_lds(wgrad_kernel<false, AOp, BOp, FM, FN>, kWgradLds, once);
+    if (!allow_lds(wgrad_kernel<false, AOp, BOp, FM, FN>, kWgradLds, once)) return MOMOE_ERR_LAUNCH;
     wgrad_kernel<false, AOp, BOp, FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
   } else {
-    allow_lds(wgrad_kernel<true, AOp, BOp, FM, FN>, kWgradLds, once_cut);
-    allow_lds(wgrad_reduce_kernel<FM, FN>, kWgradLds, once_reduce);
+    if (!allow_lds(wgrad_kernel<true, AOp, BOp, FM, FN>, kWgradLds, once_cut) ||
+        !allow_lds(wgrad_reduce_kernel<FM, FN>, kWgradLds, once_reduce))
+      return MOMOE_ERR_LAUNCH;
     wgrad_kernel<true, AOp, BOp, FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
     wgrad_reduce_kernel<FM, FN><<<grid, kThreads, kWgradLds, st>>>(a);
   }

@@ -33,6 +33,7 @@ _SIGNATURES = {
     "momoe_abi_version": (_int, []),
     "momoe_status_string": (ctypes.c_char_p, [_int]),
     "momoe_set_clock_trace": (_int, [_p]),
+    "momoe_mfma_rate_probe": (_i64, [_p, _p, _int, _p, _p]),
     "momoe_tile_table_ints": (_i64, [_i64, _i64, _i64, _int]),
     "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
     "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
@@ -112,6 +113,36 @@ class clock_trace:
         torch.cuda.synchronize()
         c, w = self.ticks.tolist()
         return 100.0 * c / w if w else float("nan")
+
+
+def mfma_rate_probe(kind="gaussian", iters=20000, launches=3):
+    """Sustained rate of the GEMMs' MFMA on register operands (momoe_mfma_rate_probe): returns
+    (TFLOP/s, shader clock in MHz).  kind: "gaussian" = N(0,1) activations against N(0,0.02)
+    weights, the layer's kind of data; "zeros"."""
+    dev = "cuda"
+    ops = torch.zeros(4096 * 8, dtype=torch.bfloat16, device=dev)
+    if kind == "gaussian":
+        g = torch.Generator(device=dev).manual_seed(5)
+        # row-side fragments come from the first half of the buffer, column-side ones from the second
+        v = torch.randn(4096, 8, generator=g, device=dev)
+        v[2048:] *= 0.02
+        ops = v.reshape(-1).to(torch.bfloat16)
+    elif kind != "zeros":
+        raise ValueError(kind)
+    sink = torch.zeros(512, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+    st = _stream()
+    flops = _lib.momoe_mfma_rate_probe(ops.data_ptr(), sink.data_ptr(), iters, ticks.data_ptr(), st)
+    if flops < 0:
+        raise RuntimeError("momoe_mfma_rate_probe failed")
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(launches):
+        _lib.momoe_mfma_rate_probe(ops.data_ptr(), sink.data_ptr(), iters, ticks.data_ptr(), st)
+    b.record()
+    torch.cuda.synchronize()
+    c, w = ticks.tolist()
+    return flops * launches / (a.elapsed_time(b) * 1e-3) / 1e12, (100.0 * c / w if w else float("nan"))
 
 
 def _call(name, *args):

@@ -19,14 +19,15 @@ from . import _hip
 # The layer requires every token to be routed to exactly K experts (momoe/momoe.py:831, the
 # reference's README) and, like the reference, does not verify it: the index build counts the
 # offending tokens on the device and reading that counter would stall the host.  With too few
-# pairs the missing contributions are simply absent from y and the gradients; with too many the
-# tile list is emptied and y is undefined.  Set CHECK_ROUTING = True to read the counter after
+# pairs the missing contributions are simply absent from y and the gradients; with too many (more
+# pairs than the M*K sorted rows) the routing is refused on the device: no GEMM runs, y and all
+# gradients are zero.  Set CHECK_ROUTING = True to read the counter after
 # every forward (one device synchronisation per call) and raise on a violation.
 CHECK_ROUTING = False
 
 # Row-tile height of the grouped GEMMs: _hip.AUTO_TILE_ROWS leaves the choice between 256 and 320
-# rows to the index build, which makes it on the device from the routing.  A fixed height (any
-# value up to _hip.TILE_ROWS) is for experiments and for tests that must cover both code paths.
+# rows to the index build, which makes it on the device from the routing.  A fixed height (a
+# multiple of 32 from 32 to _hip.TILE_ROWS) is for experiments and for tests that must cover both code paths.
 TILE_ROWS = _hip.AUTO_TILE_ROWS
 
 

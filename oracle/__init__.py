@@ -16,6 +16,8 @@ reference, which has no tests, fixtures or golden vectors of its own):
                             built from torch.nn.functional, linearity in s
 * `experts_backward_closed_form` - pinned: torch.autograd through
                             `experts_forward` in fp64 and `gradcheck`
+* `experts_forward_backward` - pinned: equals `experts_forward` and
+                            `experts_backward_closed_form` (tests/test_oracle_experts.py)
 * `router_forward`        - pinned: Ks=0/bias=0 reduces to softmax over the
                             top-k logits (library routine); brute-force top-k
 * `router_backward_closed_form` - pinned: autograd through a differentiable
@@ -33,6 +35,7 @@ from .moe_oracle import (  # noqa: F401
     experts_forward,
     experts_forward_dense,
     experts_backward_closed_form,
+    experts_forward_backward,
     router_forward,
     router_backward_closed_form,
     router_probs_differentiable,

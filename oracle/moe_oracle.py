@@ -166,7 +166,9 @@ def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
     `reference_rounding` rounds through bf16 the three intermediates that the
     reference itself stores as bf16 before they enter a weight-gradient GEMM:
     Gy' (:340, the `G_y_MsumD` buffer of :551), the recomputed h (:533-535) and
-    G_z (:527-531, `G_z_Msum2H` of :555).  Everything else stays in `dtype`.
+    G_z (:527-531, `G_z_Msum2H` of :555); the y_pre behind dL/ds is then
+    recomputed from that bf16 h, as the reference does for rows without a saved
+    y_pre (:689-697; a saved y_pre is bf16 itself).  Everything else stays in `dtype`.
     It exists to measure how far the reference's OWN arithmetic is from the
     unrounded result (tests/test_oracle_experts.py); parity tests compare
     against the unrounded form.
@@ -203,8 +205,53 @@ def experts_backward_closed_form(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD,
         G_W2[i] = rnd(h).T @ gys
         G_W1[i] = xi.T @ G_z
         G_x.index_add_(0, tok, G_z @ W1[i].T)
+        if reference_rounding:
+            ypre = rnd(h) @ W2[i]
         G_s[i, tok] = (gy * ypre).sum(dim=1)
     return G_x, G_W1, G_W2, G_s
+
+
+def experts_forward_backward(x_MD, Wl1_ND2H, Wl2_NHD, mask_NM, s_NM, G_y_MD, dtype=torch.float32):
+    """Forward and backward of the experts in one pass over the experts, every product formed
+    once: y as in `experts_forward`, the gradients as in `experts_backward_closed_form` (same
+    reference lines), with a, b, h and y_pre kept from the forward instead of recomputed -- the
+    arithmetic of the reference at save_percent=100, 18*D*H flops per (token, expert) pair.
+    No autograd: nothing but the products themselves is executed, which is what a timing of the
+    CPU path should measure.  Returns (y, G_x, G_W1, G_W2, G_s)."""
+    x = x_MD.to(dtype)
+    W1 = Wl1_ND2H.to(dtype)
+    W2 = Wl2_NHD.to(dtype)
+    s = s_NM.to(dtype)
+    Gy = G_y_MD.to(dtype)
+    N, D, H2 = W1.shape
+    H = H2 // 2
+    M = x.shape[0]
+    y = torch.zeros((M, D), dtype=dtype)
+    G_x = torch.zeros((M, D), dtype=dtype)
+    G_W1 = torch.zeros_like(W1)
+    G_W2 = torch.zeros_like(W2)
+    G_s = torch.zeros((N, M), dtype=dtype)
+    for i in range(N):
+        tok = torch.nonzero(mask_NM[i] != 0, as_tuple=False).flatten()
+        if tok.numel() == 0:
+            continue
+        xi = x.index_select(0, tok)
+        si = s[i].index_select(0, tok)[:, None]
+        z = xi @ W1[i]
+        a, b = z[:, :H], z[:, H:]
+        sig = torch.sigmoid(b)
+        h = a * b * sig
+        ypre = h @ W2[i]
+        y.index_add_(0, tok, ypre * si)
+        gy = Gy.index_select(0, tok)
+        gys = gy * si
+        G_h = gys @ W2[i].T
+        G_z = torch.cat([G_h * b * sig, G_h * a * sig * (1 + b * (1 - sig))], dim=1)
+        torch.mm(h.T, gys, out=G_W2[i])
+        torch.mm(xi.T, G_z, out=G_W1[i])
+        G_x.index_add_(0, tok, G_z @ W1[i].T)
+        G_s[i, tok] = (gy * ypre).sum(dim=1)
+    return y, G_x, G_W1, G_W2, G_s
 
 
 # --------------------------------------------------------------------------

@@ -12,14 +12,35 @@ def rel_err(got, ref):
     return ((got - ref).norm() / ref.norm().clamp_min(1e-30)).item()
 
 
+# Size of the error the cap on plain-check misses is computed for, relative to the RMS of the
+# reference: half of the norm-wise bound the same check enforces (relative L2 error < 1e-2), and
+# about twice what is measured (1.5e-3 .. 3e-3).
+MODEL_REL_ERR = 5e-3
+
+
+def _scale_of(ref):
+    if ref.dim() == 3:  # per-expert weight gradients: each expert has its own scale
+        return ref.pow(2).mean(dim=(1, 2), keepdim=True).sqrt()
+    return ref.pow(2).mean().sqrt().reshape(())
+
+
+def plain_miss_cap(ref):
+    """How many elements may miss the PLAIN rtol/atol 2e-2 check: the number a Gaussian error of
+    standard deviation MODEL_REL_ERR * rms(ref) (per expert for weight gradients) would leave
+    outside it, plus four standard deviations of that count and 2."""
+    ref = ref.detach().double().cpu()
+    sigma = (MODEL_REL_ERR * _scale_of(ref)).clamp_min(1e-30)
+    expected = torch.erfc((ATOL + RTOL * ref.abs()) / (sigma * 2 ** 0.5)).sum().item()
+    return int(expected + 4 * expected ** 0.5 + 2)
+
+
 def tolerance_report(got, ref):
     """(elements outside the plain rtol/atol 2e-2 check, elements outside the check whose
     absolute term is scaled by max(1, rms(ref)), the scale used, relative L2 error)."""
     got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
-    if ref.dim() == 3:  # per-expert weight gradients: each expert has its own scale
-        scale = ref.pow(2).mean(dim=(1, 2), keepdim=True).sqrt().clamp_min(1.0)
-    else:
-        scale = max(1.0, ref.pow(2).mean().sqrt().item())
+    scale = _scale_of(ref).clamp_min(1.0)
+    if ref.dim() != 3:
+        scale = scale.item()
     diff = (got - ref).abs()
     plain = int((diff > ATOL + RTOL * ref.abs()).sum())
     scaled = int((diff > ATOL * scale + RTOL * ref.abs()).sum())
@@ -27,27 +48,33 @@ def tolerance_report(got, ref):
 
 
 def assert_close(got, ref, what, rel=1e-2):
-    """Elementwise |got-ref| <= ATOL*max(1, rms(ref)) + RTOL*|ref| and a norm-wise bound.
+    """Elementwise |got-ref| <= ATOL*max(1, rms(ref)) + RTOL*|ref|, a norm-wise bound, and a cap
+    on the number of elements outside the plain rtol/atol 2e-2 check.
 
     For tensors whose RMS is at most 1 (y, G_x, and the weight gradients of small experts)
     this is the plain rtol/atol 2e-2 check.  The absolute term follows the RMS of larger
-    tensors (per expert for the weight gradients): the operands of the weight-gradient GEMMs
-    (G_z, h, the scaled G_y) are bf16 in the reference too (momoe/momoe.py:340, 533-535, 555),
-    their rounding accumulates over the contraction and scales with the result itself, so the
-    reference's own arithmetic misses the plain check on those tensors by the same margin
+    tensors (per expert for the weight gradients, and dL/ds): the operands of the GEMMs behind
+    them (G_z, h, the scaled G_y) are bf16 in the reference too (momoe/momoe.py:340, 533-535,
+    555, and dL/ds is formed from the bf16 h or the bf16 y_pre, :685-697), their rounding
+    accumulates over the contraction and scales with the result itself, so the reference's own
+    arithmetic misses the plain check on those tensors by the same margin
     (tests/test_oracle_experts.py::test_reference_rounding_alone_breaks_the_plain_tolerance).
-    Whenever the scaling matters, the number of elements outside the PLAIN check is printed
-    (pytest -rP / -s shows it).
+    How many elements may miss the plain check is capped (`plain_miss_cap`), so the relaxation
+    cannot drift; whenever it matters the count and the cap are printed (pytest -rP / -s).
     """
     got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
     plain, scaled, _, e = tolerance_report(got, ref)
+    cap = plain_miss_cap(ref) if plain else 0
     if plain:
-        print(f"[tolerance] {what}: {plain}/{ref.numel()} elements outside plain rtol/atol 2e-2, "
-              f"{scaled} outside the RMS-scaled check; rms(ref) {ref.pow(2).mean().sqrt().item():.3g}, "
-              f"relative L2 error {e:.2e}")
+        print(f"[tolerance] {what}: {plain}/{ref.numel()} elements outside plain rtol/atol 2e-2 "
+              f"(cap {cap}), {scaled} outside the RMS-scaled check; rms(ref) "
+              f"{ref.pow(2).mean().sqrt().item():.3g}, relative L2 error {e:.2e}")
     assert scaled == 0, (f"{what}: {scaled}/{ref.numel()} elements outside tolerance, "
                          f"max abs diff {(got - ref).abs().max().item():.4g}, rms(ref) "
                          f"{ref.pow(2).mean().sqrt().item():.4g}, relative L2 error {e:.3e}")
+    assert plain <= cap, (f"{what}: {plain}/{ref.numel()} elements outside the plain rtol/atol 2e-2 "
+                          f"check, more than the {cap} an error of {MODEL_REL_ERR:g} x rms(ref) "
+                          f"= {MODEL_REL_ERR * ref.pow(2).mean().sqrt().item():.3g} explains")
     assert e < rel, f"{what}: relative L2 error {e:.3e} >= {rel}"
 
 

@@ -138,6 +138,32 @@ def test_tokens_with_fewer_than_k_experts(sp):
     assert torch.all(dev["y"][42] == 0) and torch.all(dev["G_x"][42] == 0)
 
 
+@pytest.mark.parametrize("M,sp", [(300, 0), (300, 100), (2000, 50)])
+def test_mask_with_more_than_mk_pairs_gives_zeros(M, sp):
+    # More pairs than sorted rows exist for: the routing is refused on the device (empty tile
+    # table, violation counted).  No GEMM runs, and what is returned is defined all the same:
+    # y and every gradient are zero, never unwritten memory.
+    import momoe_amd
+    D, H, N, K = 128, 96, 8, 3
+    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, seed=6)
+    mask = mask.clone()
+    mask[:, ::2] = 1                  # every second token sits on all experts
+    s = torch.rand(N, M) * mask
+    dev = "cuda:0"
+    # poison the allocator's free blocks, which the layer's torch.empty buffers will reuse
+    junk = torch.full((64 * 2**20,), float("nan"), device=dev, dtype=torch.bfloat16)
+    del junk
+    layer = momoe_amd.MoMoE(D, H, N, K, save_percent=sp, Wl1_ND2H=W1.to(dev), Wl2_NHD=W2.to(dev))
+    xd = x.to(dev, torch.bfloat16).reshape(1, M, D).requires_grad_()
+    sd = s.to(dev).requires_grad_()
+    y, sizes = layer(xd, mask.to(dev), sd)
+    y.backward(dy.to(dev, torch.bfloat16).reshape(1, M, D))
+    torch.cuda.synchronize()
+    assert torch.equal(sizes.cpu(), (mask != 0).sum(1))
+    for t in (y, xd.grad, layer.Wl1_ND2H.grad, layer.Wl2_NHD.grad, sd.grad):
+        assert torch.all(t == 0)
+
+
 def test_opt_in_routing_check_raises():
     import momoe_amd
     from momoe_amd import experts
@@ -170,6 +196,21 @@ def test_chart_grid_harness_one_cell():
         assert res[sp]["fwd_tflops"] > 1 and res[sp]["fwd_bwd_tflops"] > 1
         saved = int(M * K * sp / 100.0) * 2 * H * 2
         assert xy + saved <= res[sp]["held_bytes"] <= xy + saved + MiB
+
+
+@pytest.mark.parametrize("M,N,K", [(12288, 64, 6), (1000, 7, 3), (64, 64, 8)])
+def test_balanced_routing_of_the_chart_harness(M, N, K):
+    # the "balanced" cells of the chart grid include one whose K does not divide N
+    # (6 x 2048 tokens, N=64, K=6): every token still gets K distinct experts and every expert
+    # floor(M*K/N) or ceil(M*K/N) tokens
+    import bench_configs
+    gen = torch.Generator(device="cuda:0").manual_seed(0)
+    mask, s = bench_configs.balanced_routing(M, N, K, gen)
+    mask, s = mask.cpu(), s.cpu()
+    assert mask.shape == (N, M) and torch.all(mask.sum(0) == K)
+    sizes = mask.sum(1)
+    assert sizes.min() >= (M * K) // N and sizes.max() <= -(-(M * K) // N)
+    assert torch.allclose(s.sum(0), torch.ones(M), atol=1e-5) and torch.all(s[mask == 0] == 0)
 
 
 @pytest.mark.parametrize("sp", [0, 50])

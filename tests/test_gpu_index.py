@@ -88,8 +88,15 @@ def test_tile_heights_no_kernel_takes_are_refused():
     with pytest.raises(RuntimeError):
         _hip.index_build(mask.to("cuda:0"), 2, tile_rows=_hip.TILE_ROWS + 32)
     ib = _hip.index_build(mask.to("cuda:0"), 2)
+    # heights below one 32-row fragment row, or not a whole number of them, would give tiles
+    # without rows: refused on the host, nothing is launched
+    for rows in (1, 16, 31, 48, 250, _hip.TILE_ROWS + 1):
+        with pytest.raises(RuntimeError):
+            _hip.index_build(mask.to("cuda:0"), 2, tile_rows=rows)
+        with pytest.raises(RuntimeError):
+            _hip.tile_table_build(ib["cumsums_N"], 300, 2, rows)
     with pytest.raises(RuntimeError):
-        _hip.tile_table_build(ib["cumsums_N"], 300, 2, _hip.TILE_ROWS + 1)
+        _hip.tile_table_build(ib["cumsums_N"], 300, 2, 0)
 
 
 def test_index_strided_mask():
