@@ -256,6 +256,12 @@ def cpu_baseline(D, H, N, K, budget_s=28.0):
             "variants": results}
 
 
+def _mark(what):
+    """Name the section that is about to use the GPU, on stderr and flushed: if a run dies there,
+    the end of its output says where."""
+    print(f"[bench] {what}", file=sys.stderr, flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -317,8 +323,10 @@ def main():
         with torch.no_grad():
             layer(xd, maskd, sd)
 
+    _mark("headline step, timed")
     layer = make_layer(args.save_percent)
     ms = timed(layer, step, args.steps, args.warmup)
+    _mark("forward only")
     ms_fwd = timed(layer, fwd_only, args.steps, 2)
     torch.cuda.reset_peak_memory_stats()
     base_mem = torch.cuda.memory_allocated()
@@ -328,6 +336,7 @@ def main():
 
     # per-kernel launch durations (HIP events on the launch stream) and the shader clock the
     # grouped GEMMs ran at (in-kernel counters), over `steps` more steps of the same loop
+    _mark("per-kernel launch times and shader clock")
     per = {}
     with _hip.clock_trace() as ct, _hip.kernel_timer() as kt:
         for _ in range(args.steps):
@@ -346,6 +355,7 @@ def main():
 
     # sustained rate: at least 2 s of back-to-back steps (the timed region above is a burst of
     # a few tens of milliseconds, and these kernels run against the power limit)
+    _mark("sustained steps")
     n_sus = max(args.steps, int(2000.0 / ms) + 1)
     with _hip.clock_trace() as ct:
         ms_sustained = timed(layer, step, n_sus, 0)
@@ -353,6 +363,7 @@ def main():
 
     # the same step captured once in a HIP graph and replayed (launch gaps only; the routing may
     # change between replays: no launch is sized from it on the host)
+    _mark("graph capture and replay")
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -366,6 +377,7 @@ def main():
     del graph
 
     # the other save setting
+    _mark("other save_percent")
     other_sp = 100 if args.save_percent == 0 else 0
     layer2 = make_layer(other_sp)
     ms_other = timed(layer2, step, max(args.steps // 2, 3), 2)
@@ -380,6 +392,7 @@ def main():
 
     # the layer with its router in front: MoE = TopKRouter -> MoMoE -> bias update
     # (momoe/sample_moe.py:59-68), gate weights ~ N(0, 1/D)
+    _mark("layer with its router")
     Wg = torch.randn(D, N, generator=torch.Generator().manual_seed(3)) / D ** 0.5
     moe = momoe_amd.MoE(D, H, N, K, 0, save_percent=args.save_percent, Wg_DN=Wg.to(dev),
                         Wl1_ND2H=layer.Wl1_ND2H.data, Wl2_NHD=layer.Wl2_NHD.data)
@@ -432,6 +445,7 @@ def main():
     # what this machine gives a plain GEMM of the up projection's size, outside the timed
     # region: the vendor library on perfectly balanced experts (no gather, no epilogue, no ragged
     # tiles), and the matrix pipe alone on register operands of the layer's kind of data
+    _mark("vendor GEMM and MFMA rate probes")
     xa = torch.randn(N, msum // N, D, device=dev).to(torch.bfloat16)
     for _ in range(3):
         torch.bmm(xa, layer.Wl1_ND2H.data)
@@ -473,6 +487,7 @@ def main():
         "roofline": roofline, "machine": machine, "kernels": kernels,
     }
     if not args.no_cpu_baseline:
+        _mark("CPU baseline (no GPU work)")
         out["cpu_baseline"] = cpu_baseline(D, H, N, K)
     print(json.dumps(out))
 

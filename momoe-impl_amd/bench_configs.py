@@ -5,6 +5,8 @@ the headline shape and prints the one JSON line the driver reads; this script pr
 
 Usage: python momoe-impl_amd/bench_configs.py            # the shapes above
        python momoe-impl_amd/bench_configs.py --only skewed   # one of: inference headline skewed large
+       python momoe-impl_amd/bench_configs.py --vendor   # the vendor GEMM library on the six GEMMs of the
+                                                         # headline step at perfectly balanced experts
        python momoe-impl_amd/bench_configs.py --chart    # the grid of the reference's README charts
                                                          # (momoe/images/moe_full.png, moe_forward.png,
                                                          # moe_memory.png): TF/s forward and
@@ -53,7 +55,7 @@ def balanced_routing(M, N, K, gen):
     return chosen.T.to(torch.int32).contiguous(), (w / w.sum(-1, keepdim=True)).contiguous().T
 
 
-def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5):
+def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5, graph=False):
     gen = torch.Generator(device=DEV).manual_seed(1)
     x = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(1, M, D)
     dy = torch.randn(M, D, generator=gen, device=DEV).to(torch.bfloat16).reshape(1, M, D)
@@ -85,6 +87,22 @@ def run(name, M, D, H, N, K, Ks=0, skew=None, sp=0, backward=True, steps=5):
     unit = float(D) * H * M * K
     tf = timeit(fwd)
     line = f"{name:30s} fwd {tf:8.3f} ms {6 * unit / tf / 1e9:6.0f} TF/s {M / tf * 1e3:11.0f} tok/s"
+    if graph:
+        # the same call captured once in a HIP graph and replayed: what a serving loop pays per
+        # call when the host does not launch kernel by kernel (no launch is sized from the routing
+        # on the host, so the replay stays valid when mask and gate weights change in place)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fwd()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fwd()
+        tg = timeit(g.replay)
+        line += f" | graph replay {tg:8.3f} ms {M / tg * 1e3:11.0f} tok/s"
+        del g
     if backward:
         torch.cuda.reset_peak_memory_stats()
         tb = timeit(step)
@@ -148,6 +166,69 @@ def chart_row(B, S, D, H, N, K, kind, steps=5):
     return result
 
 
+def vendor_gemms(D=2048, H=1024, N=128, R=512, steps=20):
+    """What the vendor GEMM library (torch.bmm) gives the six GEMMs of a step on this machine
+    when every expert holds exactly R rows: no gather, no epilogue, no ragged tiles, outputs in
+    bf16.  The figures to read this library's per-kernel times against (bench.py `kernels`): the
+    same products on the same data distribution, N(0,1) activations and N(0,0.02) weights."""
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen, device=DEV).to(torch.bfloat16)
+    x, h, gy, gz = rnd(N, R, D), rnd(N, R, H), rnd(N, R, D), rnd(N, R, 2 * H)
+    W1, W2 = rnd(N, D, 2 * H) * 0.02, rnd(N, H, D) * 0.02
+    unit = float(D) * H * R * N
+    cases = [
+        ("momoe_lin1_swiglu_fwd", f"x[{R},{D}] . Wl1[{D},{2 * H}]", 4, lambda: torch.bmm(x, W1)),
+        ("momoe_lin2_scale_fwd", f"h[{R},{H}] . Wl2[{H},{D}]", 2, lambda: torch.bmm(h, W2)),
+        ("momoe_dgrad_h", f"G_y[{R},{D}] . Wl2[{H},{D}]^T", 2, lambda: torch.bmm(gy, W2.transpose(1, 2))),
+        ("momoe_dgrad_x", f"gz[{R},{2 * H}] . Wl1[{D},{2 * H}]^T", 4, lambda: torch.bmm(gz, W1.transpose(1, 2))),
+        ("momoe_wgrad[Wl1]", f"x[{R},{D}]^T . gz[{R},{2 * H}]", 4, lambda: torch.bmm(x.transpose(1, 2), gz)),
+        ("momoe_wgrad[Wl2]", f"h[{R},{H}]^T . G_y[{R},{D}]", 2, lambda: torch.bmm(h.transpose(1, 2), gy)),
+    ]
+    print(f"torch.bmm over {N} experts of {R} rows each, bf16; ms per call and TFLOP/s", flush=True)
+    out = {}
+    for name, shape, units, fn in cases:
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        out[name] = ms
+        print(f"{name:24s} {shape:36s} {ms:7.3f} ms {units * unit / ms / 1e9:6.0f} TF/s", flush=True)
+    return out
+
+
+def read_stream_rate(gib=1.5, steps=10):
+    """GB/s at which plain library kernels read a tensor larger than the 256 MiB last-level cache
+    once (reductions over bf16 data: nothing is written back).  The figure to read the
+    weight-streaming GEMMs of the decode-sized calls against: no kernel on this machine reads HBM
+    faster than this, whatever the 8 TB/s of the data sheet say."""
+    n = int(gib * 2**30) // 2
+    t = torch.empty(n, dtype=torch.bfloat16, device=DEV).normal_()
+    ops = {"sum (fp32 accumulate)": lambda: t.sum(dtype=torch.float32), "amax": lambda: t.amax(),
+           "int32 view sum": lambda: t.view(torch.int32).sum()}
+    best = 0.0
+    for name, fn in ops.items():
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        rate = n * 2 / ms / 1e6
+        best = max(best, rate)
+        print(f"read stream, torch {name:22s} over {gib:.1f} GiB: {ms:7.3f} ms {rate:7.0f} GB/s", flush=True)
+    return best
+
+
 CHART_GRID = [
     (2, 512, 1024, 512, 32, 4, "balanced"), (4, 2048, 2048, 1024, 64, 8, "balanced"),
     (4, 2048, 2048, 1024, 64, 8, "skewed"), (6, 2048, 2048, 1280, 64, 6, "balanced"),
@@ -158,6 +239,10 @@ CHART_GRID = [
 
 if __name__ == "__main__":
     assert torch.cuda.is_available() and _hip.abi_version() == 2
+    if "--vendor" in sys.argv[1:]:
+        vendor_gemms()
+        read_stream_rate()
+        sys.exit(0)
     if "--chart" in sys.argv[1:]:
         for row in CHART_GRID:
             chart_row(*row)
@@ -165,7 +250,7 @@ if __name__ == "__main__":
     only = sys.argv[sys.argv.index("--only") + 1] if "--only" in sys.argv[1:] else None
     if only in (None, "inference"):
         for M in (16, 128, 1024, 8192):
-            run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20)
+            run(f"inference D2048 H768, M={M}", M, 2048, 768, 128, 8, backward=False, steps=20, graph=True)
     if only in (None, "headline"):
         run("headline D2048 H1024", 8192, 2048, 1024, 128, 8)
     if only in (None, "skewed"):

@@ -259,3 +259,40 @@ def test_layer_under_hip_graph_replay(sp):
         torch.cuda.synchronize()
         for name, a, b in zip(("y", "sizes", "G_x", "G_s", "G_W1", "G_W2"), captured, eager):
             assert torch.equal(a, b), (seed, name)
+
+
+def test_measurement_aids_of_the_benchmark():
+    # bench.py runs the layer under the in-kernel clock trace and the per-launch timer, and
+    # times the bare MFMA loop: the same calls at a small size, with plausible results
+    # (a shader clock between 0.5 and 3 GHz, every entry point of a step timed once per step,
+    # an MFMA rate above a tenth of the published peak).
+    import momoe_amd
+    from momoe_amd import _hip
+    M, D, H, N, K = 2048, 512, 256, 16, 4
+    dev = "cuda:0"
+    x, dy, W1, W2, mask, s = device_layer_inputs(M, D, H, N, K)
+    layer = momoe_amd.MoMoE(D, H, N, K, save_percent=0, Wl1_ND2H=W1, Wl2_NHD=W2)
+    maskd = mask.to(dev)
+
+    def step():
+        xd = x.reshape(1, M, D).clone().requires_grad_()
+        sd = s.T.contiguous().to(dev).T.requires_grad_()
+        y, _ = layer(xd, maskd, sd)
+        y.backward(dy.reshape(1, M, D))
+        layer.Wl1_ND2H.grad = layer.Wl2_NHD.grad = None
+        return y
+
+    ref = step()
+    with _hip.clock_trace() as ct, _hip.kernel_timer() as kt:
+        for _ in range(4):
+            got = step()
+    mhz = ct.mhz()
+    names = [n for n, _ in kt.durations_ms()]
+    assert 500 < mhz < 3000, mhz
+    for entry in ("momoe_index_build", "momoe_lin1_swiglu_fwd", "momoe_lin2_scale_fwd", "momoe_dgrad_h",
+                  "momoe_lin1_swiglu_bwd", "momoe_dgrad_x", "momoe_gs_scatter"):
+        assert names.count(entry) == 4, (entry, names.count(entry))
+    assert names.count("momoe_wgrad") == 8 and names.count("momoe_combine") == 8
+    assert torch.equal(got, ref)   # tracing changes no result
+    tf, clk = _hip.mfma_rate_probe("zeros", iters=2000, launches=2)
+    assert tf > 250 and 500 < clk < 3000, (tf, clk)
