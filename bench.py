@@ -442,24 +442,44 @@ def main():
                 "traffic_source": TRAFFIC_SOURCE if dom in MEASURED_TRAFFIC_BYTES else None,
                 "shader_clock_mhz": clock_timed}
 
-    # what this machine gives a plain GEMM of the up projection's size, outside the timed
-    # region: the vendor library on perfectly balanced experts (no gather, no epilogue, no ragged
-    # tiles), and the matrix pipe alone on register operands of the layer's kind of data
-    _mark("vendor GEMM and MFMA rate probes")
-    xa = torch.randn(N, msum // N, D, device=dev).to(torch.bfloat16)
-    for _ in range(3):
-        torch.bmm(xa, layer.Wl1_ND2H.data)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(10):
-        torch.bmm(xa, layer.Wl1_ND2H.data)
-    e1.record()
-    torch.cuda.synchronize()
-    vendor_ms = e0.elapsed_time(e1) / 10
-    del xa
-    machine = {"vendor_gemm_ms": vendor_ms,
-               "vendor_gemm": f"torch.bmm {N} x [{msum // N},{D}] x [{D},{2 * H}] bf16 (the flops of momoe_lin1_swiglu_fwd)",
-               "vendor_gemm_tflops": 4.0 * D * H * msum / vendor_ms / 1e9}
+    # What this machine gives outside the timed region: the vendor library on the two forward
+    # GEMMs at perfectly balanced experts (torch.bmm over N experts of Msum/N rows: no gather, no
+    # epilogue, no ragged tiles), the weight stream alone, and the matrix pipe alone on register
+    # operands of the layer's kind of data.  (Only products with untransposed operands: the
+    # batched product with a transposed weight operand of the dL/dx shape ends in an illegal
+    # memory access inside the vendor library on this software stack.)
+    def event_ms(fn, n=10):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    R = msum // N
+    gen = torch.Generator(device=dev).manual_seed(7)
+    xa = torch.randn(N, R, D, generator=gen, device=dev).to(torch.bfloat16)
+    ha = torch.randn(N, R, H, generator=gen, device=dev).to(torch.bfloat16)
+    Wa, Wb = layer.Wl1_ND2H.data, layer.Wl2_NHD.data
+    vendor = {"momoe_lin1_swiglu_fwd": lambda: torch.bmm(xa, Wa), "momoe_lin2_scale_fwd": lambda: torch.bmm(ha, Wb)}
+    machine = {"vendor_gemm": f"torch.bmm over {N} experts of {R} rows each, bf16, N(0,1) activations: x.Wl1 and h.Wl2, "
+                              "ms and TFLOP/s, and this library's launch on the real routing relative to it",
+               "vendor_gemm_ms": {}, "vendor_gemm_tflops": {}, "this_library_over_vendor": {}}
+    for k, fn in vendor.items():
+        _mark(f"vendor GEMM for {k}")
+        t = event_ms(fn)
+        machine["vendor_gemm_ms"][k] = t
+        machine["vendor_gemm_tflops"][k] = flops[k] / t / 1e9
+        machine["this_library_over_vendor"][k] = kernels[k]["avg_ms"] / t
+    del xa, ha, vendor
+    _mark("weight stream probe")
+    machine["hbm_read_stream_gbs"] = _hip.hbm_stream_probe(Wa)
+    machine["hbm_read_stream"] = (f"the grouped GEMMs' weight stream alone (global -> LDS, four 16 KiB stages per CU "
+                                  f"in flight) over Wl1, {Wa.numel() * 2 / 2**20:.0f} MiB")
+    _mark("MFMA rate probe")
     for kind in ("gaussian", "zeros"):
         tf, mhz = _hip.mfma_rate_probe(kind)
         machine[f"mfma_only_tflops_{kind}"] = tf

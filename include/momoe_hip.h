@@ -78,6 +78,17 @@ int momoe_set_clock_trace(unsigned long long* ticks2);
 int64_t momoe_mfma_rate_probe(const void* operands_64KiB, float* sink_512, int iters,
                               unsigned long long* ticks2, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the rate at which this machine streams
+ * weights from HBM when nothing else happens.  Reads `blocks` row-major bf16 matrices of
+ * krows x ncol (consecutive in memory; krows a multiple of 32, ncol of 256, one matrix below
+ * 4 GiB) exactly as the grouped GEMMs read expert weights -- global -> LDS transfers of 32 x 256
+ * stages, four stages per workgroup in flight, one workgroup per CU -- and drops the data.
+ * Returns the bytes read by the launch (time it with events on `stream`; use more bytes than
+ * the 256 MiB last-level cache holds), or -1 on a bad argument / failed launch.
+ */
+int64_t momoe_hbm_stream_probe(const void* matrix, int64_t blocks, int64_t krows, int64_t ncol,
+                               void* stream);
+
 /* ---- routing index -------------------------------------------------------
  * Replaces find_used_experts + scatter_cols_kernel (momoe/momoe.py:821-842,
  * 760-815) and the torch.sum at :830.

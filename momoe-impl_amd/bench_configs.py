@@ -5,8 +5,9 @@ the headline shape and prints the one JSON line the driver reads; this script pr
 
 Usage: python momoe-impl_amd/bench_configs.py            # the shapes above
        python momoe-impl_amd/bench_configs.py --only skewed   # one of: inference headline skewed large
-       python momoe-impl_amd/bench_configs.py --vendor   # the vendor GEMM library on the six GEMMs of the
-                                                         # headline step at perfectly balanced experts
+       python momoe-impl_amd/bench_configs.py --vendor   # the vendor GEMM library on the forward GEMMs of the
+                                                         # headline step at perfectly balanced experts, and the
+                                                         # rate at which library kernels read HBM
        python momoe-impl_amd/bench_configs.py --chart    # the grid of the reference's README charts
                                                          # (momoe/images/moe_full.png, moe_forward.png,
                                                          # moe_memory.png): TF/s forward and
@@ -167,22 +168,23 @@ def chart_row(B, S, D, H, N, K, kind, steps=5):
 
 
 def vendor_gemms(D=2048, H=1024, N=128, R=512, steps=20):
-    """What the vendor GEMM library (torch.bmm) gives the six GEMMs of a step on this machine
-    when every expert holds exactly R rows: no gather, no epilogue, no ragged tiles, outputs in
-    bf16.  The figures to read this library's per-kernel times against (bench.py `kernels`): the
-    same products on the same data distribution, N(0,1) activations and N(0,0.02) weights."""
+    """What the vendor GEMM library (torch.bmm) gives the two forward GEMMs of a step on this
+    machine when every expert holds exactly R rows: no gather, no epilogue, no ragged tiles,
+    outputs in bf16.  The figures to read this library's per-kernel times against (bench.py
+    `kernels`): the same products on the same data distribution, N(0,1) activations and
+    N(0,0.02) weights.
+    Only the products with untransposed operands are timed.  The transposed ones (the data and
+    weight gradients) are left out on purpose: on this image the batched product
+    gz[128,512,2048] . Wl1[128,2048,2048]^T ends in an illegal memory access inside the vendor
+    library (no kernel of this repository involved) and takes the GPU down with it."""
     gen = torch.Generator(device=DEV).manual_seed(0)
     rnd = lambda *shape: torch.randn(*shape, generator=gen, device=DEV).to(torch.bfloat16)
-    x, h, gy, gz = rnd(N, R, D), rnd(N, R, H), rnd(N, R, D), rnd(N, R, 2 * H)
+    x, h = rnd(N, R, D), rnd(N, R, H)
     W1, W2 = rnd(N, D, 2 * H) * 0.02, rnd(N, H, D) * 0.02
     unit = float(D) * H * R * N
     cases = [
         ("momoe_lin1_swiglu_fwd", f"x[{R},{D}] . Wl1[{D},{2 * H}]", 4, lambda: torch.bmm(x, W1)),
         ("momoe_lin2_scale_fwd", f"h[{R},{H}] . Wl2[{H},{D}]", 2, lambda: torch.bmm(h, W2)),
-        ("momoe_dgrad_h", f"G_y[{R},{D}] . Wl2[{H},{D}]^T", 2, lambda: torch.bmm(gy, W2.transpose(1, 2))),
-        ("momoe_dgrad_x", f"gz[{R},{2 * H}] . Wl1[{D},{2 * H}]^T", 4, lambda: torch.bmm(gz, W1.transpose(1, 2))),
-        ("momoe_wgrad[Wl1]", f"x[{R},{D}]^T . gz[{R},{2 * H}]", 4, lambda: torch.bmm(x.transpose(1, 2), gz)),
-        ("momoe_wgrad[Wl2]", f"h[{R},{H}]^T . G_y[{R},{D}]", 2, lambda: torch.bmm(h.transpose(1, 2), gy)),
     ]
     print(f"torch.bmm over {N} experts of {R} rows each, bf16; ms per call and TFLOP/s", flush=True)
     out = {}

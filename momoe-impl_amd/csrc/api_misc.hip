@@ -64,8 +64,44 @@ __global__ __launch_bounds__(kThreads, 2) void mfma_rate_kernel(const u32x4* __r
     ticks2[1] = wall_clock64() - w0;
   }
 }
+// Nothing but the weight stream of the grouped GEMMs: global -> LDS transfers of [32 k-rows] x
+// [256 columns] stages of a row-major matrix, a ring of four stages per workgroup, one workgroup
+// per CU walking (matrix, column block) tiles; nothing reads the data.
+__global__ __launch_bounds__(kThreads) void hbm_stream_kernel(const bf16* __restrict__ w, int64_t blocks,
+                                                              int krows, int ncol) {
+  constexpr int S = 4;
+  TDma B;
+  const uint32_t lds = lds_address(dyn_lds());
+  const int nb = ncol / TLayout::COLS, ktiles = krows / kBK;
+  for (int64_t t = blockIdx.x; t < blocks * nb; t += gridDim.x) {
+    const int64_t e = t / nb;
+    const int tn = (int)(t % nb);
+    B.init(w + e * krows * ncol, [&](int c) { return tn * TLayout::COLS + c; }, ncol);
+    for (int s = 0; s < S - 1 && s < ktiles; ++s) B.issue(s, lds + s * (TLayout::LDS_ELEMS * 2));
+    for (int kt = 0; kt < ktiles; ++kt) {
+      if (kt + S - 1 < ktiles) {
+        B.issue(kt + S - 1, lds + ((kt + S - 1) % S) * (TLayout::LDS_ELEMS * 2));
+        wait_vmcnt<(S - 1) * TDma::NCH>();
+      } else {
+        wait_vmcnt<0>();
+      }
+      __builtin_amdgcn_s_barrier();
+    }
+  }
+}
 }  // namespace
 }  // namespace momoe
+
+extern "C" int64_t momoe_hbm_stream_probe(const void* matrix, int64_t blocks, int64_t krows,
+                                          int64_t ncol, void* stream) {
+  if (!matrix || blocks <= 0 || krows <= 0 || ncol <= 0 || ((uintptr_t)matrix & 15)) return -1;
+  if (krows % momoe::kBK != 0 || ncol % momoe::TLayout::COLS != 0 || krows * ncol * 2 >= (1ll << 32))
+    return -1;
+  momoe::hbm_stream_kernel<<<momoe::persistent_grid(), momoe::kThreads, 4 * momoe::TLayout::LDS_ELEMS * 2,
+                             (hipStream_t)stream>>>((const momoe::bf16*)matrix, blocks, (int)krows, (int)ncol);
+  if (hipGetLastError() != hipSuccess) return -1;
+  return blocks * krows * ncol * 2;
+}
 
 extern "C" int64_t momoe_mfma_rate_probe(const void* operands_64KiB, float* sink_512, int iters,
                                          unsigned long long* ticks2, void* stream) {

@@ -32,6 +32,11 @@ constexpr int kTileHeader = 4;
 // position of the first sorted row `row0` of expert `e` (momoe_padded_rows() bounds them all):
 __host__ __device__ __forceinline__ int padded_start(int row0, int e) { return ((row0 + 31) & ~31) + 32 * e; }
 
+// Index of this wavefront in its workgroup, as a value the compiler knows to be the same in every
+// lane: what is derived from it (the rows and columns a wave owns, its share of a transfer) then
+// lives in scalar registers instead of taking a vector register per value.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 struct TileCoord {
   int expert;  // expert index
   int row0;    // first sorted row of this tile
@@ -122,7 +127,7 @@ struct TileSched {
     tc.rows = min(32 * (fbase + (tl < fextra ? 1 : 0)), r.mi - 32 * f0);
     // the tile's fragment rows are dealt to the two wave rows as evenly as possible
     const int nf = (tc.rows + 31) >> 5, half = (nf + 1) >> 1;
-    const bool upper = threadIdx.x >= 256;
+    const bool upper = wave_id() >= kWaves / 2;
     tc.mbase = upper ? 32 * half : 0;
     tc.na = upper ? nf - half : half;
     return tc;

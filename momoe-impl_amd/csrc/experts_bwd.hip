@@ -75,7 +75,7 @@ __device__ __forceinline__ void dgrad_h_tiles(const DhArgs& p) {
   using Prog = DhProg<G>;
   typename Prog::Ring ring(dyn_lds());
   TileSched sched(p.table, (p.H + BN - 1) / BN, G::MAX_ROWS);
-  const int wn = (threadIdx.x >> 6) & 3;
+  const int wn = wave_id() & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   Prog prog{p, p.D / kBK, wn};
   run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);
@@ -249,7 +249,7 @@ __device__ __forceinline__ void dgrad_x_tiles(const DxArgs& p) {
   using Prog = DxProg<G>;
   typename Prog::Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN, G::MAX_ROWS);
-  const int wn = (threadIdx.x >> 6) & 3;
+  const int wn = wave_id() & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   Prog prog{p, (2 * p.H) / kBK, wn};
   run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);

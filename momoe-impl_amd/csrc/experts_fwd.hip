@@ -258,7 +258,7 @@ __device__ __forceinline__ void lin1_swiglu_tiles(const Lin1Args& p) {
   const int first_tile =
       p.h == nullptr && p.ab_lo > 0 ? TileSched::expert_tile_of_row(p.table, p.ab_lo) : 0;
   TileSched sched(p.table, (p.H + Prog::BNH - 1) / Prog::BNH, Prog::BM, first_tile);
-  const int wn = (threadIdx.x >> 6) & 3;
+  const int wn = wave_id() & 3;
   const int n_org[FN] = {wn * 32, Prog::BNH + wn * 32};
   Prog prog{p, p.D / kBK, wn};
   run_row_tiles<FM, FN>(prog, sched, ring, n_org);
@@ -348,7 +348,7 @@ __device__ __forceinline__ void lin2_scale_tiles(const Lin2Args& p) {
   using Prog = Lin2Prog<G>;
   typename Prog::Ring ring(dyn_lds());
   TileSched sched(p.table, (p.D + BN - 1) / BN, G::MAX_ROWS);
-  const int wn = (threadIdx.x >> 6) & 3;
+  const int wn = wave_id() & 3;
   const int n_org[FN] = {wn * 64, wn * 64 + 32};
   Prog prog{p, p.H / kBK, wn};
   run_row_tiles<Prog::FM, FN>(prog, sched, ring, n_org);

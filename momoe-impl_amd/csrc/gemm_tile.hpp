@@ -131,7 +131,7 @@ struct RDma {
 
   // tile row whose piece this lane fetches in deposit j
   static __device__ __forceinline__ int row_of(int j) {
-    return (j * kWaves + (threadIdx.x >> 6)) * 16 + ((threadIdx.x & 63) >> 2);
+    return (j * kWaves + wave_id()) * 16 + ((threadIdx.x & 63) >> 2);
   }
   // row r of the tile starts at (char*)base_ + rowoff(r, j), j being the deposit that fetches
   // it for this lane (r = row_of(j)); every r < ROWS must be readable
@@ -147,7 +147,7 @@ struct RDma {
     }
   }
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
-    const int w = threadIdx.x >> 6;
+    const int w = wave_id();
     const bf16* b = base + kt * kBK;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) dma16(b, off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
@@ -181,7 +181,7 @@ struct RBlockedDma {
     r.init(mat + row0 * kBK, [&](int row, int) { return (uint32_t)min(row, nvalid - 1) * (uint32_t)(kBK * 2); });
   }
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
-    const int w = threadIdx.x >> 6;
+    const int w = wave_id();
     const bf16* b = r.base + (int64_t)kt * kstride;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) dma16(b, r.off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
@@ -206,12 +206,12 @@ struct TLayout {
 
   // k-row and logical column (multiple of 8) fetched by this lane in deposit j
   static __device__ __forceinline__ void lane_piece(int j, int& krow, int& col) {
-    const int l = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int l = threadIdx.x & 63, w = wave_id();
     krow = w * (2 * NCH) + j * 2 + (l >> 5);
     col = ((l & 31) ^ swz(krow)) * 8;
   }
   static __device__ __forceinline__ uint32_t deposit(uint32_t stage, int j) {
-    return stage + ((threadIdx.x >> 6) * NCH + j) * (kChunkElems * 2);
+    return stage + (wave_id() * NCH + j) * (kChunkElems * 2);
   }
   // 32 columns starting at c0 (multiple of 32), k-step kk (16 k-values)
   static __device__ __forceinline__ bf16x8 frag(const bf16* stage, int c0, int kk) {
@@ -298,7 +298,7 @@ struct TGatherDmaT {
 
   // sorted row behind k-row j of this wave's deposits in stage kt
   __device__ __forceinline__ int row_of(int kt, int j) const {
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int w = wave_id();
     return min(row_begin + kt * kBK + w * kRows + j, row_end - 1);
   }
   // start the scalar loads of the ids of stage kt; the results must not be touched before
@@ -720,16 +720,23 @@ struct RowStager {
   static constexpr int CHUNKS = 4 * NF;        // 16-byte chunks per staged row
   static constexpr int PITCH = 32 * NF;        // elements per staged row
   static constexpr int PASSES = 32 * CHUNKS / 64;
+  // The 16-byte chunks of a staged row are permuted by the row: the 64 banks hold 256 bytes, i.e.
+  // 256 / (2 * PITCH) consecutive rows, so the permutation must change from one such group of
+  // rows to the next for the 32 rows x 8 bytes that the two half-waves put() at a time to spread
+  // over all banks (two passes, the least 512 bytes take).  Permuting by the row itself left
+  // rows 8 (4) apart on the same banks: four (eight) passes.
+  static constexpr int ROWS_PER_BANK_ROW = 256 / (2 * PITCH);
+  static __device__ __forceinline__ int swz(int row) { return (row / ROWS_PER_BANK_ROW) & (CHUNKS - 1); }
   bf16* st;  // this wave's staging area
 
   // `slot` selects one of the 2/NF staging areas of this wave
   __device__ __forceinline__ explicit RowStager(bf16* epilogue_lds, int slot = 0)
-      : st(epilogue_lds + (threadIdx.x >> 6) * (kStageBytesPerWave / 2) + slot * (32 * PITCH)) {}
+      : st(epilogue_lds + wave_id() * (kStageBytesPerWave / 2) + slot * (32 * PITCH)) {}
 
   // this lane's quad q of fragment f: row lane%32, columns 32f + 8q + 4*(lane/32) .. +3
   __device__ __forceinline__ void put(int f, int q, bf16x4 v) const {
     const int l = threadIdx.x & 63, row = l & 31, half = l >> 5;
-    const int c = (4 * f + q) ^ (row & (CHUNKS - 1));
+    const int c = (4 * f + q) ^ swz(row);
     *(bf16x4*)(st + row * PITCH + c * 8 + half * 4) = v;
   }
   // pass p of PASSES: 16 bytes = columns [col, col+8) of row `row` (both relative to the
@@ -738,7 +745,7 @@ struct RowStager {
     const int l = threadIdx.x & 63;
     row = p * (64 / CHUNKS) + l / CHUNKS;
     const int pc = l % CHUNKS;
-    col = (pc ^ (row & (CHUNKS - 1))) * 8;
+    col = (pc ^ swz(row)) * 8;
     return *(const bf16x8*)(st + row * PITCH + pc * 8);
   }
   // write everything put() since the last flush: dst(row, col) -> destination of 8 columns,

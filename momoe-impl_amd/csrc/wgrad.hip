@@ -82,7 +82,7 @@ struct TransposedOperand {
            [&](int row, int) { return (uint32_t)min(row, nfeat - 1 - f0) * 64u; });
   }
   __device__ __forceinline__ void issue(int kt, uint32_t stage) {
-    const int w = threadIdx.x >> 6;
+    const int w = wave_id();
     const bf16* b = r.base + (int64_t)kt * gstride;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) dma16(b, r.off[j], stage + (j * kWaves + w) * (kChunkElems * 2));
@@ -124,7 +124,7 @@ struct WaveTile {
   static constexpr int WAVES_N = 256 / (32 * FN);  // waves side by side
   int m_org[FM], n_org[FN];
   __device__ __forceinline__ WaveTile() {
-    const int wave = threadIdx.x >> 6, wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int wave = wave_id(), wm = wave / WAVES_N, wn = wave % WAVES_N;
 #pragma unroll
     for (int i = 0; i < FM; ++i) m_org[i] = wm * (32 * FM) + 32 * i;
 #pragma unroll
@@ -289,7 +289,7 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 // A partial tile is kept in accumulator order: per wave, per fragment, 4 x (64 lanes x 16 B).
 template <int FM, int FN>
 __device__ __forceinline__ f32x4* partial_piece(float* ws, int slot, int i, int f, int qd) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = wave_id(), lane = threadIdx.x & 63;
   return (f32x4*)(ws + (int64_t)slot * (BX * BY)) +
          ((((wave * FM + i) * FN + f) * 4 + qd) * 64 + lane);
 }

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "momoe_status_string": (ctypes.c_char_p, [_int]),
     "momoe_set_clock_trace": (_int, [_p]),
     "momoe_mfma_rate_probe": (_i64, [_p, _p, _int, _p, _p]),
+    "momoe_hbm_stream_probe": (_i64, [_p, _i64, _i64, _i64, _p]),
     "momoe_tile_table_ints": (_i64, [_i64, _i64, _i64, _int]),
     "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
     "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
@@ -143,6 +144,24 @@ def mfma_rate_probe(kind="gaussian", iters=20000, launches=3):
     torch.cuda.synchronize()
     c, w = ticks.tolist()
     return flops * launches / (a.elapsed_time(b) * 1e-3) / 1e12, (100.0 * c / w if w else float("nan"))
+
+
+def hbm_stream_probe(weights_NKC, launches=5):
+    """GB/s at which the weight stream of the grouped GEMMs alone reads the bf16 tensor
+    [blocks, krows, ncol] (momoe_hbm_stream_probe); give it more than the last-level cache holds."""
+    blocks, krows, ncol = weights_NKC.shape
+    st = _stream()
+    args = (weights_NKC.data_ptr(), blocks, krows, ncol, st)
+    nbytes = _lib.momoe_hbm_stream_probe(*args)
+    if nbytes < 0:
+        raise RuntimeError("momoe_hbm_stream_probe failed")
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(launches):
+        _lib.momoe_hbm_stream_probe(*args)
+    b.record()
+    torch.cuda.synchronize()
+    return nbytes * launches / (a.elapsed_time(b) * 1e-3) / 1e9
 
 
 def _call(name, *args):
