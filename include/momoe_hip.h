@@ -267,7 +267,10 @@ int momoe_dgrad_x(const void* gz_blocked, const void* Wl1_ND2H, const int32_t* t
  *                            At most one operand may be transposed.
  *   MOMOE_LAYOUT_KBLOCKED    (B only) bf16 [features/32][ld][32] with ld >= Msum = rows of the
  *                            matrix, no gather: B(r, y) = B[((y / 32) * ld + r) * 32 + y % 32];
- *                            Y a multiple of 32.  This is how gz is written.
+ *                            Y a multiple of 32.  This is how gz is written.  The eight
+ *                            32-column blocks of a tile are addressed with 32-bit byte offsets:
+ *                            8 * ld * 64 bytes must stay below 4 GiB, i.e. ld < 8 388 608 rows
+ *                            (about one million tokens at K = 8), else MOMOE_ERR_UNSUPPORTED.
  * M = number of tokens (rows of a gathered matrix, and the most rows an expert can hold);
  * M * ld * 2 bytes (row layout) must stay below 4 GiB.  Experts without rows get exact zeros.
  * Wl2 gradient: A = hs (transposed, X=H), B = G_y gathered by idx (Y=D).

@@ -204,31 +204,16 @@ def vendor_gemms(D=2048, H=1024, N=128, R=512, steps=20):
     return out
 
 
-def read_stream_rate(gib=1.5, steps=10):
-    """GB/s at which plain library kernels read a tensor larger than the 256 MiB last-level cache
-    once (reductions over bf16 data: nothing is written back).  The figure to read the
-    weight-streaming GEMMs of the decode-sized calls against: no kernel on this machine reads HBM
-    faster than this, whatever the 8 TB/s of the data sheet say."""
-    n = int(gib * 2**30) // 2
-    t = torch.empty(n, dtype=torch.bfloat16, device=DEV).normal_()
-    ops = {"sum (fp32 accumulate)": lambda: t.sum(dtype=torch.float32), "amax": lambda: t.amax(),
-           "int32 view sum": lambda: t.view(torch.int32).sum()}
-    best = 0.0
-    for name, fn in ops.items():
-        for _ in range(2):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / steps
-        rate = n * 2 / ms / 1e6
-        best = max(best, rate)
-        print(f"read stream, torch {name:22s} over {gib:.1f} GiB: {ms:7.3f} ms {rate:7.0f} GB/s", flush=True)
-    return best
+def read_stream_rate(gib=1.5):
+    """GB/s at which the weight stream of the grouped GEMMs alone (global -> LDS transfers, nothing
+    else: momoe_hbm_stream_probe) reads a tensor larger than the 256 MiB last-level cache.  The
+    figure to read the weight-streaming GEMMs of the decode-sized calls against: it is what this
+    machine delivers to that access pattern, whatever the 8 TB/s of the data sheet say."""
+    blocks = int(gib * 2**30) // (2048 * 2048 * 2)
+    w = torch.empty((blocks, 2048, 2048), dtype=torch.bfloat16, device=DEV).normal_()
+    rate = _hip.hbm_stream_probe(w)
+    print(f"weight stream alone over {blocks * 8} MiB: {rate:7.0f} GB/s", flush=True)
+    return rate
 
 
 CHART_GRID = [

@@ -72,9 +72,14 @@ class MoEFunction(torch.autograd.Function):
             mask = mask_NM.to(device=dev, dtype=torch.int32)
             s = s_NM.to(device=dev, dtype=torch.float32)
 
+            msum = M * K
+            # the Wl1 gradient addresses the eight 32-column blocks of a gz tile with 32-bit byte
+            # offsets (momoe_wgrad, k-blocked operand): say so now rather than in the backward
+            if ctx.needs_input_grad[1] and 8 * msum * 64 >= 2 ** 32:
+                raise RuntimeError(f"MoMoE backward supports fewer than 8388608 (token, expert) pairs per call, "
+                                   f"got {msum}: split the batch")
             ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS)
             idx, table = ib["idx_Msum"], ib["tile_table"]
-            msum = M * K
             # nothing is kept for a backward that cannot happen (no input wants a gradient)
             msave = _saved_rows(msum, save_percent) if any(ctx.needs_input_grad[:5]) else 0
 

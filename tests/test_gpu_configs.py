@@ -296,3 +296,20 @@ def test_measurement_aids_of_the_benchmark():
     assert torch.equal(got, ref)   # tracing changes no result
     tf, clk = _hip.mfma_rate_probe("zeros", iters=2000, launches=2)
     assert tf > 250 and 500 < clk < 3000, (tf, clk)
+
+
+def test_backward_row_limit_is_reported_in_the_forward():
+    # the Wl1 gradient takes fewer than 8 388 608 (token, expert) pairs per call (32-bit offsets
+    # into the k-blocked gz): a larger training batch is refused before anything is launched,
+    # not in the backward after the forward succeeded
+    import momoe_amd
+    D, H, N, K = 32, 32, 8, 8
+    M = 2 ** 20
+    dev = "cuda:0"
+    layer = momoe_amd.MoMoE(D, H, N, K)
+    x = torch.zeros(1, M, D, device=dev, dtype=torch.bfloat16)
+    mask = torch.ones(N, M, device=dev, dtype=torch.int32)
+    s = torch.full((N, M), 1.0 / N, device=dev)
+    with pytest.raises(RuntimeError, match="8388608"):
+        layer(x, mask, s)
+    del x, mask, s
