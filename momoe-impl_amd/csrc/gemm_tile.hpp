@@ -720,6 +720,13 @@ struct RowStager {
   static constexpr int CHUNKS = 4 * NF;        // 16-byte chunks per staged row
   static constexpr int PITCH = 32 * NF;        // elements per staged row
   static constexpr int PASSES = 32 * CHUNKS / 64;
+  // The 16-byte chunks of a staged row are permuted by the row: the 64 banks hold 256 bytes, i.e.
+  // 256 / (2 * PITCH) consecutive rows, so the permutation must change from one such group of
+  // rows to the next for the 32 rows x 8 bytes that the two half-waves put() at a time to spread
+  // over all banks (two passes, the least 512 bytes take).  Permuting by the row itself left
+  // rows 8 (4) apart on the same banks: four (eight) passes.
+  static constexpr int ROWS_PER_BANK_ROW = 256 / (2 * PITCH);
+  static __device__ __forceinline__ int swz(int row) { return (row / ROWS_PER_BANK_ROW) & (CHUNKS - 1); }
   bf16* st;  // this wave's staging area
 
   // `slot` selects one of the 2/NF staging areas of this wave
@@ -729,7 +736,7 @@ struct RowStager {
   // this lane's quad q of fragment f: row lane%32, columns 32f + 8q + 4*(lane/32) .. +3
   __device__ __forceinline__ void put(int f, int q, bf16x4 v) const {
     const int l = threadIdx.x & 63, row = l & 31, half = l >> 5;
-    const int c = (4 * f + q) ^ (row & (CHUNKS - 1));
+    const int c = (4 * f + q) ^ swz(row);
     *(bf16x4*)(st + row * PITCH + c * 8 + half * 4) = v;
   }
   // pass p of PASSES: 16 bytes = columns [col, col+8) of row `row` (both relative to the
@@ -738,7 +745,7 @@ struct RowStager {
     const int l = threadIdx.x & 63;
     row = p * (64 / CHUNKS) + l / CHUNKS;
     const int pc = l % CHUNKS;
-    col = (pc ^ (row & (CHUNKS - 1))) * 8;
+    col = (pc ^ swz(row)) * 8;
     return *(const bf16x8*)(st + row * PITCH + pc * 8);
   }
   // write everything put() since the last flush: dst(row, col) -> destination of 8 columns,
