@@ -720,11 +720,12 @@ struct RowStager {
   static constexpr int CHUNKS = 4 * NF;        // 16-byte chunks per staged row
   static constexpr int PITCH = 32 * NF;        // elements per staged row
   static constexpr int PASSES = 32 * CHUNKS / 64;
-  // The 16-byte chunks of a staged row are permuted by the row: the 64 banks hold 256 bytes, i.e.
-  // 256 / (2 * PITCH) consecutive rows, so the permutation must change from one such group of
-  // rows to the next for the 32 rows x 8 bytes that the two half-waves put() at a time to spread
-  // over all banks (two passes, the least 512 bytes take).  Permuting by the row itself left
-  // rows 8 (4) apart on the same banks: four (eight) passes.
+  // The 16-byte chunks of a staged row are permuted by the row.  The 64 banks hold 256 bytes, i.e.
+  // 256 / (2 * PITCH) consecutive rows, so the permutation changes from one such group of rows to
+  // the next: the 32 rows x 8 bytes that a half-wave put()s at a time then spread over the banks.
+  // Measured (SQ_LDS_BANK_CONFLICT per launch of the headline layer): with 64-byte rows (NF = 1,
+  // the x.Wl1 kernels) a third of what permuting by the row itself gave (3.4 M -> 1.1 M forward,
+  // 6.5 M -> 2.2 M backward); with 128-byte rows (NF = 2) no change, 1024 cycles per tile.
   static constexpr int ROWS_PER_BANK_ROW = 256 / (2 * PITCH);
   static __device__ __forceinline__ int swz(int row) { return (row / ROWS_PER_BANK_ROW) & (CHUNKS - 1); }
   bf16* st;  // this wave's staging area
