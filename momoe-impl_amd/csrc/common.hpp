@@ -100,7 +100,10 @@ struct TileSched {
     r.any = true;
     return r;
   }
-  __device__ __forceinline__ TileCoord resolve(const Raw& r) const {
+  __device__ __forceinline__ TileCoord resolve(const Raw& r) const { return resolve_raw(r, nb, bm); }
+  // the arithmetic of resolve() for a table entry however it was obtained: nb column blocks,
+  // tiles of at most bm rows
+  static __device__ __forceinline__ TileCoord resolve_raw(const Raw& r, int nb, int bm) {
     TileCoord tc;
     tc.valid = r.any;
     if (!r.any) return tc;
