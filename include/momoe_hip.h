@@ -165,24 +165,6 @@ int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H, const int32_t*
                           void* ab_rows, int64_t ab_row_lo, int64_t ab_row_hi,
                           int64_t M, int64_t D, int64_t H, int64_t N, int64_t Msum, void* stream);
 
-/* momoe_lin1_swiglu_fwd_small: momoe_index_build and momoe_lin1_swiglu_fwd in ONE launch, for
- * decode-sized calls: M <= 256 tokens, N <= 256 experts, M*K <= 4096 pairs (else
- * MOMOE_ERR_UNSUPPORTED: make the two calls).  Replaces find_used_experts + scatter_cols_kernel
- * (momoe/momoe.py:821-842, 760-815) and lin1_kernel (:69-152) together.  Every workgroup builds
- * the routing index of the call in its own LDS and walks its tiles from there, so the GEMM does
- * not wait for a separate index launch (17-19 us of a 160-230 us call); workgroup 0 also writes
- * the index outputs to memory, bit-identical to momoe_index_build's with tile_rows = 256, for the
- * kernels that follow (momoe_lin2_scale_fwd, momoe_combine, the backward).  Arguments: those of
- * the two calls (no workspace: the build needs none); violations as in momoe_index_build.
- */
-int momoe_lin1_swiglu_fwd_small(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m,
-                                const void* x_MD, const void* Wl1_ND2H,
-                                int64_t* sizes_N, int32_t* cumsums_N1, int32_t* idx_Msum,
-                                int32_t* which_Msum, int32_t* inv_MK, int32_t* tile_table,
-                                int32_t* violations, void* h_blocked,
-                                void* ab_rows, int64_t ab_row_lo, int64_t ab_row_hi,
-                                int64_t M, int64_t D, int64_t H, int64_t N, int64_t K, void* stream);
-
 /* momoe_lin2_scale_fwd replaces lin2_kernel (momoe/momoe.py:161-237):
  *   ys[r] = bf16( (h[r] @ Wl2[i]) * s[i, idx[r]] ), rows kept in sorted order.
  * h_blocked as written by momoe_lin1_swiglu_fwd.

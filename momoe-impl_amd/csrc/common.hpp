@@ -100,10 +100,7 @@ struct TileSched {
     r.any = true;
     return r;
   }
-  __device__ __forceinline__ TileCoord resolve(const Raw& r) const { return resolve_raw(r, nb, bm); }
-  // the arithmetic of resolve() for a table entry however it was obtained: nb column blocks,
-  // tiles of at most bm rows
-  static __device__ __forceinline__ TileCoord resolve_raw(const Raw& r, int nb, int bm) {
+  __device__ __forceinline__ TileCoord resolve(const Raw& r) const {
     TileCoord tc;
     tc.valid = r.any;
     if (!r.any) return tc;

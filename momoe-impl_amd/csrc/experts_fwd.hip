@@ -4,7 +4,6 @@
 #include <type_traits>
 
 #include "gemm_tile.hpp"
-#include "index_small.hpp"
 
 namespace momoe {
 namespace {
@@ -32,17 +31,7 @@ struct Lin1Args {
   float* gs_part;
   int64_t msum;
   unsigned long long* clk;
-  // small calls only (token ids come from the index the workgroup built in LDS): that index, and
-  // the number of tokens, which ids read from it are clamped to
-  const int32_t* lds_idx;
-  int ntok;
 };
-
-// int32 from LDS through the LDS port (a generic load would also count as a vector-memory
-// operation, which the hand-counted waits on the transfers do not expect)
-__device__ __forceinline__ int32_t lds_load_i32(const int32_t* p) {
-  return *(const int32_t __attribute__((address_space(3)))*)p;
-}
 
 // Tile = up to 320 (256) rows x (128 `a` columns + the matching 128 `b` columns); a wave owns 32 `a`
 // columns and their 32 `b` columns, so the SwiGLU product pairs registers of the same lane.
@@ -50,11 +39,9 @@ __device__ __forceinline__ int32_t lds_load_i32(const int32_t* p) {
 // stay in registers and go straight into the SwiGLU backward.
 // G: the row-tile geometry.  The forward takes either; the backward's epilogue needs the registers
 // of the fifth fragment row, so it only exists for 256-row tiles and runs on a tile table of its own.
-// LDSIDX: the token of a sorted row is read from p.lds_idx (LDS) instead of p.idx (forward only).
-template <bool BWD, class G, bool LDSIDX = false>
+template <bool BWD, class G>
 struct Lin1Prog {
   static_assert(!BWD || std::is_same_v<G, StdTiles>, "the SwiGLU backward epilogue fits 256-row tiles only");
-  static_assert(!(BWD && LDSIDX), "the small-call path is forward only");
   static constexpr int FM = G::FM, BM = G::MAX_ROWS;
   using RowsOp = RDma<G::AROWS>;  // token rows, k-contiguous
   using Ring = StageRing<RowsOp, WeightOp, G::STAGES>;
@@ -72,10 +59,7 @@ struct Lin1Prog {
 
   __device__ __forceinline__ void gather(const TileCoord& t, Prep& g) const {
 #pragma unroll
-    for (int j = 0; j < RowsOp::NCH; ++j) {
-      const int r = t.row0 + min(RowsOp::row_of(j), t.rows - 1);
-      g.tok[j] = LDSIDX ? min(max(lds_load_i32(p.lds_idx + r), 0), p.ntok - 1) : p.idx[r];
-    }
+    for (int j = 0; j < RowsOp::NCH; ++j) g.tok[j] = p.idx[t.row0 + min(RowsOp::row_of(j), t.rows - 1)];
     if (BWD) {
 #pragma unroll
       for (int i = 0; i < FM; ++i) g.etok[i] = p.idx[t.row0 + min(t.mbase + 32 * i + acc_row(), t.rows - 1)];
@@ -295,96 +279,6 @@ __global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_kernel(Lin1Args p) {
 constexpr size_t kLin1FwdLds = std::max(Lin1Prog<false, TallTiles>::kLds, Lin1Prog<false, StdTiles>::kLds);
 constexpr size_t kLin1BwdLds = Lin1Prog<true, StdTiles>::kLds;
 
-// ---- x.Wl1 for decode-sized calls: the routing index is built by the kernel itself ----------------
-// At most 256 tokens and 256 experts.  Every workgroup builds the index of the call in its own
-// LDS (index_small.hpp: a few microseconds, against a whole dependent launch before the GEMM can
-// start) and walks its tiles from there; workgroup 0 also writes the index to memory, where the
-// kernels after this one (h.Wl2, the combine, the backward) find it exactly as momoe_index_build
-// would have left it.  One row tile per expert: no expert holds more than 256 rows.
-struct SmallIndexArgs {
-  const int32_t* mask;
-  int64_t sn, sm;
-  int M, N, K;
-  int64_t* sizes;
-  int32_t* cumsums;
-  int32_t* idx;
-  int32_t* which;
-  int32_t* inv;
-  int32_t* table;
-  int32_t* violations;
-};
-
-// Tile iterator over the experts that hold a token, read from the index in LDS: the same walk as
-// TileSched (id%8 = XCD, each XCD a contiguous eighth of the expert-major tile sequence, its
-// workgroups striding through it).
-template <int NGROUPS>
-struct LdsSched {
-  using Raw = TileSched::Raw;
-  const int32_t* cum;  // LDS
-  const int32_t* act;  // LDS
-  int nb, nexp, total, chunk, xcd, pos, stride;
-  __device__ __forceinline__ LdsSched(const SmallIndexLds<NGROUPS>& L, int nb_, int nexp_)
-      : cum(L.cum), act(L.act), nb(nb_), nexp(nexp_) {
-    total = __builtin_amdgcn_readfirstlane(lds_load_i32(&L.nact)) * nb;
-    chunk = (total + 7) >> 3;
-    xcd = blockIdx.x & 7;
-    pos = blockIdx.x >> 3;
-    stride = gridDim.x >> 3;
-  }
-  __device__ __forceinline__ Raw fetch() {
-    Raw r;
-    r.any = false;
-    if (pos >= chunk) return r;
-    const int q = xcd * chunk + pos;
-    pos += stride;
-    if (q >= total) return r;
-    const int a = q / nb;  // a < nact <= experts of the build: inside `act`
-    const int e = min(max(__builtin_amdgcn_readfirstlane(lds_load_i32(act + a)), 0), nexp - 1);
-    const int c0 = __builtin_amdgcn_readfirstlane(lds_load_i32(cum + e));
-    const int c1 = __builtin_amdgcn_readfirstlane(lds_load_i32(cum + e + 1));
-    r.q = q;
-    r.expert = e;
-    r.first = a;  // one row tile per expert: the expert's first tile is its place among the active ones
-    r.rstart = c0;
-    r.mi = min(max(c1 - c0, 1), MOMOE_RECOMPUTE_TILE_ROWS);
-    r.any = true;
-    return r;
-  }
-  __device__ __forceinline__ TileCoord resolve(const Raw& r) const {
-    return TileSched::resolve_raw(r, nb, MOMOE_RECOMPUTE_TILE_ROWS);
-  }
-  __device__ __forceinline__ TileCoord next() { return resolve(fetch()); }
-};
-
-constexpr int kSmallMaxPairs = 4096;  // sorted rows whose tokens the LDS copy of the index holds
-template <int NGROUPS>
-constexpr size_t small_index_lds_bytes() {
-  return (sizeof(SmallIndexLds<NGROUPS>) + 1023) / 1024 * 1024 + (size_t)kSmallMaxPairs * sizeof(int32_t);
-}
-using SmallLin1Prog = Lin1Prog<false, StdTiles, true>;
-constexpr size_t kLin1SmallLds = SmallLin1Prog::kLds + small_index_lds_bytes<kSmallMaxGroups>();
-static_assert(kLin1SmallLds <= 160 * 1024, "ring and index fit the CU's LDS");
-
-template <int NGROUPS>
-__global__ __launch_bounds__(kThreads, 2) void lin1_swiglu_small_kernel(Lin1Args p, SmallIndexArgs q) {
-  const ClockTrace trace(p.clk);
-  using Ring = typename SmallLin1Prog::Ring;
-  char* lds = (char*)dyn_lds();
-  SmallIndexLds<NGROUPS>& L = *(SmallIndexLds<NGROUPS>*)(lds + Ring::BYTES);
-  int32_t* lds_idx = (int32_t*)(lds + Ring::BYTES + (sizeof(SmallIndexLds<NGROUPS>) + 1023) / 1024 * 1024);
-  const SmallIndexOut out{q.sizes, q.cumsums, q.idx, q.which, q.inv, q.table, q.violations, blockIdx.x == 0};
-  small_index_build<NGROUPS>(q.mask, q.sn, q.sm, q.M, q.N, q.K, 0, L, lds_idx, out);
-  p.lds_idx = lds_idx;
-  p.ntok = q.M;
-  Ring ring(dyn_lds());
-  LdsSched<NGROUPS> sched(L, (p.H + SmallLin1Prog::BNH - 1) / SmallLin1Prog::BNH, q.N);
-  const int wn = wave_id() & 3;
-  const int n_org[FN] = {wn * 32, SmallLin1Prog::BNH + wn * 32};
-  SmallLin1Prog prog{p, p.D / kBK, wn};
-  run_row_tiles<SmallLin1Prog::FM, FN>(prog, sched, ring, n_org);
-  trace.finish();
-}
-
 struct Lin2Args {
   const bf16* h;
   const bf16* w2;
@@ -536,42 +430,6 @@ extern "C" int momoe_lin1_swiglu_fwd(const void* x_MD, const void* Wl1_ND2H,
   static LdsLimit lds;
   if (!allow_lds(lin1_swiglu_kernel<false>, kLin1FwdLds, lds)) return MOMOE_ERR_LAUNCH;
   lin1_swiglu_kernel<false><<<persistent_grid(), kThreads, kLin1FwdLds, (hipStream_t)stream>>>(a);
-  return launch_status();
-}
-
-extern "C" int momoe_lin1_swiglu_fwd_small(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m,
-                                           const void* x_MD, const void* Wl1_ND2H, int64_t* sizes_N,
-                                           int32_t* cumsums_N1, int32_t* idx_Msum, int32_t* which_Msum,
-                                           int32_t* inv_MK, int32_t* tile_table, int32_t* violations,
-                                           void* h_blocked, void* ab_rows, int64_t ab_row_lo,
-                                           int64_t ab_row_hi, int64_t M, int64_t D, int64_t H, int64_t N,
-                                           int64_t K, void* stream) {
-  if (!mask_NM || !x_MD || !Wl1_ND2H || !sizes_N || !cumsums_N1 || !idx_Msum || !which_Msum || !inv_MK ||
-      !tile_table || !violations || (!h_blocked && !ab_rows))
-    return MOMOE_ERR_BAD_ARG;
-  if (!aligned16(x_MD) || !aligned16(Wl1_ND2H) || ((uintptr_t)h_blocked & 15) || ((uintptr_t)ab_rows & 15))
-    return MOMOE_ERR_BAD_ARG;
-  if (K <= 0) return MOMOE_ERR_BAD_ARG;
-  const int st = check_dims(M, D, H, N, M * K);
-  if (st != MOMOE_OK) return st;
-  // what one workgroup indexes: one token panel, the experts of the one-workgroup build, and as
-  // many pairs as the LDS copy of the index holds
-  if (M > kPanelTokens || N > kSmallMaxExperts || M * K > kSmallMaxPairs) return MOMOE_ERR_UNSUPPORTED;
-  Lin1Args a{(const bf16*)x_MD, (const bf16*)Wl1_ND2H, idx_Msum, tile_table, (bf16*)h_blocked,
-             (bf16*)ab_rows, ab_row_lo, ab_row_hi, (int)D, (int)H,
-             nullptr, nullptr, 0, 0, nullptr, nullptr, 0, nullptr, M * K, clock_trace_buffer(), nullptr, (int)M};
-  SmallIndexArgs q{mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N, cumsums_N1, idx_Msum,
-                   which_Msum, inv_MK, tile_table, violations};
-  hipStream_t s = (hipStream_t)stream;
-  if (N <= 128) {
-    static LdsLimit lds;
-    if (!allow_lds(lin1_swiglu_small_kernel<8>, kLin1SmallLds, lds)) return MOMOE_ERR_LAUNCH;
-    lin1_swiglu_small_kernel<8><<<persistent_grid(), kThreads, kLin1SmallLds, s>>>(a, q);
-  } else {
-    static LdsLimit lds;
-    if (!allow_lds(lin1_swiglu_small_kernel<kSmallMaxGroups>, kLin1SmallLds, lds)) return MOMOE_ERR_LAUNCH;
-    lin1_swiglu_small_kernel<kSmallMaxGroups><<<persistent_grid(), kThreads, kLin1SmallLds, s>>>(a, q);
-  }
   return launch_status();
 }
 

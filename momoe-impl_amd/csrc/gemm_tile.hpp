@@ -666,9 +666,8 @@ constexpr size_t kEpilogueLds = (size_t)kWaves * kStageBytesPerWave;
 // While tile t is multiplied: the table entry of tile t+2 and the gathered values of tile t+1
 // are in flight; after its main loop the first stages of tile t+1 are requested, then the
 // epilogue of tile t runs.
-// Sched: TileSched, or anything with its fetch() / resolve() / next() and Raw.
-template <int FM, int FN, class P, class Sched, class AOp, class BOp, int NS>
-__device__ __forceinline__ void run_row_tiles(P& prog, Sched& sched, StageRing<AOp, BOp, NS>& ring,
+template <int FM, int FN, class P, class AOp, class BOp, int NS>
+__device__ __forceinline__ void run_row_tiles(P& prog, TileSched& sched, StageRing<AOp, BOp, NS>& ring,
                                               const int (&n_org)[FN]) {
   static_assert(StageRing<AOp, BOp, NS>::STAGE * sizeof(bf16) >= kEpilogueLds, "a stage buffer holds the store staging");
   TileCoord c0 = sched.next();
@@ -684,7 +683,7 @@ __device__ __forceinline__ void run_row_tiles(P& prog, Sched& sched, StageRing<A
   while (true) {
     f32x16 acc[FN][FM];
     zero_acc<FM, FN>(acc);
-    typename Sched::Raw rn;
+    TileSched::Raw rn;
     int m_org[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) m_org[i] = c0.mbase + 32 * i;

@@ -14,12 +14,31 @@
 #include <mutex>
 
 #include "common.hpp"
-#include "index_small.hpp"
 
 namespace momoe {
 namespace {
 
+constexpr int kPanelTokens = 256;
+constexpr int kPanelExperts = 16;
 constexpr int kMaxExperts = 4096;
+
+// The 16 mask entries of token m in expert group g, as a bit set.  Loads are unconditional (row
+// and column clamped into the matrix, the result masked afterwards): a load under a branch is
+// waited for before the next one is issued, which made this function one memory latency PER
+// ENTRY instead of one per group.
+__device__ __forceinline__ uint32_t load_panel_bits(const int32_t* __restrict__ mask, int64_t sn,
+                                                    int64_t sm, int M, int N, int g, int m) {
+  const int32_t* col = mask + (int64_t)min(m, M - 1) * sm;
+  int32_t v[kPanelExperts];
+#pragma unroll
+  for (int e = 0; e < kPanelExperts; ++e)
+    v[e] = col[(int64_t)min(g * kPanelExperts + e, N - 1) * sn];
+  uint32_t bits = 0;
+#pragma unroll
+  for (int e = 0; e < kPanelExperts; ++e)
+    bits |= (v[e] != 0 && g * kPanelExperts + e < N ? 1u : 0u) << e;
+  return m < M ? bits : 0u;
+}
 
 __global__ __launch_bounds__(kPanelTokens) void index_count_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int NC,
@@ -40,6 +59,15 @@ __global__ __launch_bounds__(kPanelTokens) void index_count_kernel(
     const int i = g * kPanelExperts + t;
     if (i < N) part[(int64_t)i * NC + c] = wcnt[t][0] + wcnt[t][1] + wcnt[t][2] + wcnt[t][3];
   }
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int o = __shfl_up(v, d);
+    if (lane >= d) v += o;
+  }
+  return v;
 }
 
 // Tile height for a routing (tile_rows = 0 asked for it).  A row tile streams its rows and a
@@ -190,16 +218,107 @@ __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
 
 // The whole index build in one launch of one workgroup, for at most 256 tokens (one token
 // panel) and 256 experts: decode-sized calls, where three dependent launches cost more than
-// the work (index_small.hpp).
+// the work.  Thread t is token t and reads its whole mask column up front (all loads in flight
+// at once: one memory latency), as 16 bits per group of 16 experts; one ballot per expert gives
+// the lane masks of its tokens, a scan over the experts gives cumsums and the tile table, and
+// every token then places its own K pairs from its bits and those masks.
+constexpr int kSmallMaxGroups = 16;
+constexpr int kSmallMaxExperts = kSmallMaxGroups * kPanelExperts;
+
 template <int NGROUPS>
 __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
     int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
     int tile_rows_arg, int32_t* __restrict__ violations) {
-  __shared__ SmallIndexLds<NGROUPS> lds;
-  const SmallIndexOut out{sizes, cumsums, idx, which, inv, table, violations, true};
-  small_index_build<NGROUPS>(mask, sn, sm, M, N, K, tile_rows_arg, lds, nullptr, out);
+  // asked to choose the tile height: with at most 256 tokens no expert holds more than 256 rows,
+  // and taller tiles save nothing
+  const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
+  static_assert(kPanelTokens <= MOMOE_RECOMPUTE_TILE_ROWS, "one tile per expert in the one-launch kernel");
+  __shared__ uint64_t ball[NGROUPS * kPanelExperts][4];  // tokens of expert i in wave w, as a lane mask
+  __shared__ int32_t s_cum[NGROUPS * kPanelExperts];
+  __shared__ int32_t s_wave[4][2];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int64_t msum = (int64_t)M * K;
+  uint32_t bits[NGROUPS];
+#pragma unroll
+  for (int g = 0; g < NGROUPS; ++g) bits[g] = load_panel_bits(mask, sn, sm, M, N, g, t);
+#pragma unroll
+  for (int g = 0; g < NGROUPS; ++g)
+#pragma unroll
+    for (int e = 0; e < kPanelExperts; ++e) {
+      const uint64_t b = __ballot((bits[g] >> e) & 1u);
+      if (lane == 0) ball[g * kPanelExperts + e][wave] = b;
+    }
+  __syncthreads();
+  // exclusive scan over the experts of (rows, row tiles): one expert per thread
+  const int v = t < N ? __popcll(ball[t][0]) + __popcll(ball[t][1]) + __popcll(ball[t][2]) + __popcll(ball[t][3]) : 0;
+  const int nt = (v + tile_rows - 1) / tile_rows;
+  const int irows = wave_inclusive_scan(v, lane), itiles = wave_inclusive_scan(nt, lane);
+  if (lane == 63) {
+    s_wave[wave][0] = irows;
+    s_wave[wave][1] = itiles;
+  }
+  __syncthreads();
+  int brow = irows - v, btile = itiles - nt;
+  for (int w = 0; w < wave; ++w) {
+    brow += s_wave[w][0];
+    btile += s_wave[w][1];
+  }
+  const int total = s_wave[0][0] + s_wave[1][0] + s_wave[2][0] + s_wave[3][0];
+  const int total_tiles = s_wave[0][1] + s_wave[1][1] + s_wave[2][1] + s_wave[3][1];
+  const bool overflow = (int64_t)total > msum;
+  if (t < NGROUPS * kPanelExperts) s_cum[t] = brow;
+  if (t < N) {
+    cumsums[t] = brow;
+    sizes[t] = (int64_t)v;
+    if (!overflow)
+      for (int k = 0; k < nt; ++k) {
+        int32_t* e = table + kTileHeader + 4 * (btile + k);
+        e[0] = t;
+        e[1] = btile;
+        e[2] = brow;
+        e[3] = v;
+      }
+  }
+  if (t == 0) {
+    cumsums[N] = total;
+    if (overflow) atomicAdd(violations, 1);
+    table[0] = overflow ? 0 : total_tiles;
+    table[1] = tile_rows;
+    table[2] = 0;
+    table[3] = 0;
+  }
+  // sorted rows past the last pair (a routing with fewer than M*K pairs): token 0, slot 0
+  for (int64_t r = (int64_t)total + t; r < msum; r += kPanelTokens) {
+    idx[r] = 0;
+    which[r] = 0;
+  }
+  __syncthreads();
+  // every token walks its own pairs (K of them, not N candidates), lowest expert first
+  const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int k = 0;
+#pragma unroll
+  for (int g = 0; g < NGROUPS; ++g) {
+    uint32_t rest = bits[g];
+    while (rest != 0) {
+      const int i = g * kPanelExperts + __ffs(rest) - 1;
+      rest &= rest - 1;
+      int before = __popcll(ball[i][wave] & below);
+      for (int w = 0; w < wave; ++w) before += __popcll(ball[i][w]);
+      const int64_t row = (int64_t)s_cum[i] + before;
+      if (row < msum) {
+        idx[row] = t;
+        which[row] = k;
+      }
+      if (k < K) inv[(int64_t)t * K + k] = row < msum && !overflow ? (int32_t)row : -1;
+      ++k;
+    }
+  }
+  if (t < M && k != K) {
+    atomicAdd(violations, 1);
+    for (int kk = k; kk < K; ++kk) inv[(int64_t)t * K + kk] = -1;
+  }
 }
 
 // A tile table for another tile height from the prefix sums of a finished index build.

@@ -44,8 +44,6 @@ _SIGNATURES = {
                                         _int, _p, _p]),
     "momoe_lin1_swiglu_fwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64,
                                      _i64, _p]),
-    "momoe_lin1_swiglu_fwd_small": (_int, [_p, _i64, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64,
-                                           _i64, _i64, _i64, _i64, _i64, _i64, _p]),
     "momoe_lin2_scale_fwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64,
                                     _i64, _p]),
     "momoe_combine": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _p]),
@@ -248,41 +246,6 @@ def lin1_swiglu_fwd(x_MD, Wl1_ND2H, idx, table, h, ab, ab_lo, ab_hi):
     _call("momoe_lin1_swiglu_fwd", _ptr(x_MD), _ptr(Wl1_ND2H), _ptr(idx), _ptr(table), _ptr(h),
                                       _ptr(ab), ab_lo, ab_hi, M, D, H2 // 2, N, idx.numel(),
                                       _stream())
-
-
-SMALL_MAX_TOKENS = 256   # what momoe_lin1_swiglu_fwd_small takes: one token panel,
-SMALL_MAX_EXPERTS = 256  # the experts of the one-workgroup index build,
-SMALL_MAX_PAIRS = 4096   # and the pairs whose tokens the LDS copy of the index holds
-
-
-def small_call(M, N, K):
-    """Whether a call of M tokens, N experts, K experts per token fits the one-launch
-    index + x.Wl1 kernel for decode-sized calls."""
-    return M <= SMALL_MAX_TOKENS and N <= SMALL_MAX_EXPERTS and M * K <= SMALL_MAX_PAIRS
-
-
-def lin1_swiglu_fwd_small(mask_NM, K, x_MD, Wl1_ND2H, h, ab, ab_lo, ab_hi):
-    """Routing index and x.Wl1 + SwiGLU in one launch (momoe_lin1_swiglu_fwd_small); returns the
-    same dict as index_build (256-row tile table)."""
-    _need_cuda(mask_NM, x_MD, Wl1_ND2H)
-    assert mask_NM.dtype == torch.int32 and mask_NM.dim() == 2
-    N, M = mask_NM.shape
-    D = x_MD.shape[1]
-    H2 = Wl1_ND2H.shape[2]
-    dev = mask_NM.device
-    msum = M * K
-    sizes = torch.empty(N, dtype=torch.int64, device=dev)
-    cumsums = torch.empty(N + 1, dtype=torch.int32, device=dev)
-    idx = torch.empty(msum, dtype=torch.int32, device=dev)
-    which = torch.empty(msum, dtype=torch.int32, device=dev)
-    inv = torch.empty(msum, dtype=torch.int32, device=dev)
-    table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, RECOMPUTE_TILE_ROWS), dtype=torch.int32, device=dev)
-    violations = torch.zeros(1, dtype=torch.int32, device=dev)
-    _call("momoe_lin1_swiglu_fwd_small", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), _ptr(x_MD),
-          _ptr(Wl1_ND2H), _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv), _ptr(table),
-          _ptr(violations), _ptr(h), _ptr(ab), ab_lo, ab_hi, M, D, H2 // 2, N, K, _stream())
-    return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
-            "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
 
 
 def lin2_scale_fwd(h, Wl2_NHD, s_NM, idx, table, ys, M):

@@ -30,11 +30,6 @@ CHECK_ROUTING = False
 # multiple of 32 from 32 to _hip.TILE_ROWS) is for experiments and for tests that must cover both code paths.
 TILE_ROWS = _hip.AUTO_TILE_ROWS
 
-# Calls of at most 256 tokens, 256 experts and 4096 (token, expert) pairs build their routing index
-# inside the up projection's kernel (one launch fewer in front of the first GEMM).  False: always
-# the separate index build (for tests that compare the two).
-SMALL_CALLS = True
-
 
 def _saved_rows(msum, save_percent):
     # momoe/momoe.py:251
@@ -83,19 +78,15 @@ class MoEFunction(torch.autograd.Function):
             if ctx.needs_input_grad[1] and 8 * msum * 64 >= 2 ** 32:
                 raise RuntimeError(f"MoMoE backward supports fewer than 8388608 (token, expert) pairs per call, "
                                    f"got {msum}: split the batch")
+            ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS)
+            idx, table = ib["idx_Msum"], ib["tile_table"]
             # nothing is kept for a backward that cannot happen (no input wants a gradient)
             msave = _saved_rows(msum, save_percent) if any(ctx.needs_input_grad[:5]) else 0
+
             # h in blocks of 32 hidden columns, [H/32][Msum][32]: the layout the down projection reads
             h = torch.empty((H // 32, msum, 32), device=dev, dtype=torch.bfloat16)
             ab_save = torch.empty((msave, 2 * H), device=dev, dtype=torch.bfloat16) if msave > 0 else None
-            if SMALL_CALLS and TILE_ROWS in (_hip.AUTO_TILE_ROWS, _hip.RECOMPUTE_TILE_ROWS) and _hip.small_call(M, N, K):
-                # decode-sized call: the up projection builds the routing index itself
-                ib = _hip.lin1_swiglu_fwd_small(mask, K, x_MD, W1, h, ab_save, 0, msave)
-                idx, table = ib["idx_Msum"], ib["tile_table"]
-            else:
-                ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS)
-                idx, table = ib["idx_Msum"], ib["tile_table"]
-                _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, h, ab_save, 0, msave)
+            _hip.lin1_swiglu_fwd(x_MD, W1, idx, table, h, ab_save, 0, msave)
             ys = torch.empty((msum, D), device=dev, dtype=torch.bfloat16)
             _hip.lin2_scale_fwd(h, W2, s, idx, table, ys, M)
             del h

@@ -313,25 +313,3 @@ def test_backward_row_limit_is_reported_in_the_forward():
     with pytest.raises(RuntimeError, match="8388608"):
         layer(x, mask, s)
     del x, mask, s
-
-
-@pytest.mark.parametrize("M,N,K,sp", [(16, 128, 8, 0), (128, 128, 8, 100), (200, 24, 5, 50)])
-def test_small_calls_match_the_two_launch_path_bit_for_bit(M, N, K, sp):
-    # decode-sized calls build their index inside the up projection's kernel: forward and
-    # backward must not differ from the separate index build in a single bit
-    import momoe_amd
-    from momoe_amd import experts
-    D, H = 256, 160
-    x, W1, W2, mask, s, dy = make_layer_inputs(M, D, H, N, K, seed=12)
-    assert experts.SMALL_CALLS
-    a = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
-    experts.SMALL_CALLS = False
-    try:
-        b = run_device_layer(x, W1, W2, mask, s, dy, K, sp)
-    finally:
-        experts.SMALL_CALLS = True
-    for k in a:
-        assert torch.equal(a[k], b[k]), k
-    ref = run_oracle_layer(x, W1, W2, mask, s, dy)
-    for k in ("y", "G_x", "G_W1", "G_W2", "G_s"):
-        assert_close(a[k], ref[k], k)

@@ -169,67 +169,3 @@ def test_routing_with_missing_pairs_leaves_nothing_undefined():
     assert np.array_equal(out["which_Msum"].numpy()[:total], o["which_Msum"])
     assert np.all(out["idx_Msum"].numpy()[total:] == 0) and np.all(out["which_Msum"].numpy()[total:] == 0)
     assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])  # the oracle writes -1 for missing pairs
-
-
-def _run_fused(mask, K, D=64, H=32):
-    """The index as the one-launch index + x.Wl1 kernel for decode-sized calls writes it
-    (momoe_lin1_swiglu_fwd_small), together with the h it produced."""
-    from momoe_amd import _hip
-    N, M = mask.shape
-    dev = "cuda:0"
-    g = torch.Generator().manual_seed(M * 131 + N)
-    x = torch.randn(M, D, generator=g).to(dev, torch.bfloat16)
-    W1 = (torch.randn(N, D, 2 * H, generator=g) * 0.1).to(dev, torch.bfloat16)
-    h = torch.full((H // 32, M * K, 32), float("nan"), device=dev, dtype=torch.bfloat16)
-    out = _hip.lin1_swiglu_fwd_small(mask.to(dev), K, x, W1, h, None, 0, 0)
-    torch.cuda.synchronize()
-    return {k: v.cpu() for k, v in out.items()}, x, W1, h
-
-
-@pytest.mark.parametrize("M,N,K,Ks,skew", [
-    (1, 4, 4, 0, None), (16, 128, 8, 0, None), (128, 128, 8, 0, None), (256, 128, 8, 0, None),
-    (200, 200, 7, 2, None), (255, 256, 6, 0, 1.8), (77, 17, 17, 0, None), (256, 16, 16, 0, None),
-])
-def test_fused_small_call_index_is_the_index_build(M, N, K, Ks, skew):
-    # the kernel that builds the index itself must leave in memory exactly what
-    # momoe_index_build leaves (256-row tile table), and the h of the plain kernel
-    from momoe_amd import _hip
-    mask, _ = make_routing(M, N, K, Ks, seed=21, skew=skew)
-    out, x, W1, h = _run_fused(mask, K)
-    ref = _hip.index_build(mask.to("cuda:0"), K, tile_rows=_hip.RECOMPUTE_TILE_ROWS)
-    for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum", "inv_MK", "violations"):
-        assert torch.equal(out[k], ref[k].cpu()), k
-    o = oracle.index_build(mask)
-    nt = int(out["tile_table"][0])
-    assert torch.equal(out["tile_table"][:4 + 4 * nt], ref["tile_table"].cpu()[:4 + 4 * nt])
-    _check_table(out["tile_table"].numpy(), o, _hip.RECOMPUTE_TILE_ROWS)
-    h2 = torch.full_like(h, float("nan"))
-    _hip.lin1_swiglu_fwd(x, W1, ref["idx_Msum"], ref["tile_table"], h2, None, 0, 0)
-    torch.cuda.synchronize()
-    assert torch.equal(h.view(torch.int16), h2.view(torch.int16))   # bit for bit, unwritten rows included
-
-
-def test_fused_small_call_with_broken_routings():
-    from momoe_amd import _hip
-    mask, _ = make_routing(100, 40, 4, seed=4)
-    bad = mask.clone()
-    bad[:, 5] = 0          # token 5 has no expert
-    bad[0:6, 9] = 1        # token 9 has more than K
-    bad[7] = 0             # an expert without tokens
-    out, _, _, _ = _run_fused(bad, 4)
-    ref = {k: v.cpu() for k, v in _hip.index_build(bad.to("cuda:0"), 4, tile_rows=256).items()}
-    for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum", "inv_MK", "violations"):
-        assert torch.equal(out[k], ref[k]), k
-    assert out["violations"].item() >= 2
-    # too many pairs in total: refused, nothing is multiplied, every token points nowhere
-    over = torch.ones(40, 100, dtype=torch.int32)
-    out, _, _, h = _run_fused(over, 4)
-    assert out["violations"].item() >= 1 and out["tile_table"][0].item() == 0
-    assert torch.all(out["inv_MK"] == -1) and torch.isnan(h.float()).all()
-    # shapes past what one workgroup indexes go to the two-call path
-    big, _ = make_routing(300, 8, 2, seed=1)
-    with pytest.raises(RuntimeError, match="unsupported"):
-        _run_fused(big, 2)
-    wide, _ = make_routing(256, 32, 17, seed=1)   # 256 x 17 pairs > 4096
-    with pytest.raises(RuntimeError, match="unsupported"):
-        _run_fused(wide, 17)
