@@ -321,6 +321,108 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
   }
 }
 
+// The same for at most 64 tokens, the other way round: thread e is EXPERT e and holds its row of
+// the mask as a 64-bit set of tokens.  Transposing the mask costs one ballot per token here (at
+// most 64) instead of one per expert (128 to 256 in the kernel above, whose 17 us are mostly that,
+// serial in every wavefront): a 16-token call has its index in a quarter of the time.
+// MCH = ceil(M / 16): all of a thread's mask loads are in flight at once.
+constexpr int kTinyTokens = 64;
+template <int MCH>
+__global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
+    const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
+    int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
+    int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
+    int tile_rows_arg, int32_t* __restrict__ violations) {
+  static_assert(MCH >= 1 && 16 * MCH <= kTinyTokens, "token chunks of 16");
+  const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
+  __shared__ uint64_t tokb[kTinyTokens][4];  // experts of token m among the experts of wave w, as a lane mask
+  __shared__ int32_t s_wave[4][2];
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  const int64_t msum = (int64_t)M * K;
+  // the expert's row of the mask as a bit set; loads unconditional, row and column clamped
+  uint64_t bits = 0;
+  {
+    const int32_t* row = mask + (int64_t)min(e, N - 1) * sn;
+    int32_t v[16 * MCH];
+#pragma unroll
+    for (int m = 0; m < 16 * MCH; ++m) v[m] = row[(int64_t)min(m, M - 1) * sm];
+#pragma unroll
+    for (int m = 0; m < 16 * MCH; ++m) bits |= (uint64_t)(v[m] != 0 && m < M ? 1 : 0) << m;
+    if (e >= N) bits = 0;
+  }
+  // per token: the experts that hold it
+  for (int m = 0; m < M; ++m) {
+    const uint64_t b = __ballot((bits >> m) & 1ull);
+    if (lane == 0) tokb[m][wave] = b;
+  }
+  // exclusive scan over the experts of (rows, row tiles)
+  const int v = __popcll(bits);
+  const int nt = (v + tile_rows - 1) / tile_rows;
+  const int irows = wave_inclusive_scan(v, lane), itiles = wave_inclusive_scan(nt, lane);
+  if (lane == 63) {
+    s_wave[wave][0] = irows;
+    s_wave[wave][1] = itiles;
+  }
+  __syncthreads();
+  int brow = irows - v, btile = itiles - nt;
+  for (int w = 0; w < wave; ++w) {
+    brow += s_wave[w][0];
+    btile += s_wave[w][1];
+  }
+  const int total = s_wave[0][0] + s_wave[1][0] + s_wave[2][0] + s_wave[3][0];
+  const int total_tiles = s_wave[0][1] + s_wave[1][1] + s_wave[2][1] + s_wave[3][1];
+  const bool overflow = (int64_t)total > msum;
+  if (e < N) {
+    cumsums[e] = brow;
+    sizes[e] = (int64_t)v;
+    if (!overflow)
+      for (int k = 0; k < nt; ++k) {
+        int32_t* t = table + kTileHeader + 4 * (btile + k);
+        t[0] = e;
+        t[1] = btile;
+        t[2] = brow;
+        t[3] = v;
+      }
+  }
+  if (e == 0) {
+    cumsums[N] = total;
+    if (overflow) atomicAdd(violations, 1);
+    table[0] = overflow ? 0 : total_tiles;
+    table[1] = tile_rows;
+    table[2] = 0;
+    table[3] = 0;
+  }
+  // sorted rows past the last pair (a routing with fewer than M*K pairs): token 0, slot 0
+  for (int64_t r = (int64_t)total + e; r < msum; r += kPanelTokens) {
+    idx[r] = 0;
+    which[r] = 0;
+  }
+  // the expert places its pairs, lowest token first; the slot of a pair within its token is the
+  // number of lower-numbered experts that hold the token
+  const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  uint64_t rest = bits;
+  for (int r = 0; rest != 0; ++r) {
+    const int m = __ffsll((unsigned long long)rest) - 1;
+    rest &= rest - 1;
+    int k = __popcll(tokb[m][wave] & below);
+    for (int w = 0; w < wave; ++w) k += __popcll(tokb[m][w]);
+    const int64_t srow = (int64_t)brow + r;
+    if (srow < msum) {
+      idx[srow] = m;
+      which[srow] = k;
+    }
+    if (k < K) inv[(int64_t)m * K + k] = srow < msum && !overflow ? (int32_t)srow : -1;
+  }
+  // tokens whose pair count is not K: thread m looks after token m
+  if (e < M) {
+    const int k = __popcll(tokb[e][0]) + __popcll(tokb[e][1]) + __popcll(tokb[e][2]) + __popcll(tokb[e][3]);
+    if (k != K) {
+      atomicAdd(violations, 1);
+      for (int kk = k; kk < K; ++kk) inv[(int64_t)e * K + kk] = -1;
+    }
+  }
+}
+
 // A tile table for another tile height from the prefix sums of a finished index build.
 __global__ __launch_bounds__(1024) void tile_table_kernel(const int32_t* __restrict__ cumsums, int N,
                                                           int64_t msum_cap, int tile_rows,
@@ -415,6 +517,14 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
   int32_t* part = (int32_t*)workspace;
   int32_t* tokcnt = part + N * NC;
   hipStream_t st = (hipStream_t)stream;
+  if (M <= kTinyTokens && N <= kPanelTokens) {
+    auto kernel = M <= 16 ? index_tiny_kernel<1> : M <= 32 ? index_tiny_kernel<2>
+                : M <= 48 ? index_tiny_kernel<3> : index_tiny_kernel<4>;
+    kernel<<<1, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N,
+                                       cumsums_N1, idx_Msum, which_Msum, inv_MK, tile_table,
+                                       tile_rows, violations);
+    return launch_status();
+  }
   if (NC == 1 && N <= kSmallMaxExperts) {
     auto kernel = N <= 128 ? index_small_kernel<8> : index_small_kernel<kSmallMaxGroups>;
     kernel<<<1, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N,

@@ -66,6 +66,13 @@ def _compare(mask, K, out):
     (255, 1024, 6, 0, 1.8),     # many experts, few tokens
     (256, 1025, 3, 0, None),    # N one past a multiple of the 16-expert panel
     (77, 17, 17, 0, None),      # every token on every expert, N just over one group
+    # at most 64 tokens and 256 experts: the kernel with one thread per expert
+    (64, 256, 8, 0, None),      # its largest case
+    (33, 17, 17, 0, None),      # every token on every expert
+    (48, 200, 7, 2, None),      # two shared experts, experts in all four wavefronts
+    (17, 255, 6, 0, 1.8),       # skewed, one token past a chunk of 16
+    (64, 257, 4, 0, None),      # one expert too many for it: the one-panel kernel
+    (65, 256, 4, 0, None),      # one token too many
 ])
 def test_index_bit_exact(M, N, K, Ks, skew):
     mask, _ = make_routing(M, N, K, Ks, seed=11, skew=skew)
@@ -169,3 +176,35 @@ def test_routing_with_missing_pairs_leaves_nothing_undefined():
     assert np.array_equal(out["which_Msum"].numpy()[:total], o["which_Msum"])
     assert np.all(out["idx_Msum"].numpy()[total:] == 0) and np.all(out["which_Msum"].numpy()[total:] == 0)
     assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])  # the oracle writes -1 for missing pairs
+
+
+def test_violations_strides_and_missing_pairs_with_one_thread_per_expert():
+    # the same checks at 64 tokens or fewer, where another kernel builds the index
+    from momoe_amd import _hip
+    M, N, K = 40, 130, 4
+    mask, _ = make_routing(M, N, K, seed=5)
+    strided = mask.T.contiguous().to("cuda:0").T  # strides (1, N)
+    _compare(mask, K, {k: v.cpu() for k, v in _hip.index_build(strided, K).items()})
+    bad = mask.clone()
+    bad[:, 5] = 0          # token 5 has no expert
+    bad[0:6, 9] = 1        # token 9 has more than K
+    out = _run(bad, K)
+    assert out["violations"].item() >= 2
+    over = torch.ones(N, M, dtype=torch.int32)
+    out = _run(over, K)
+    assert out["violations"].item() >= 1 and out["tile_table"][0].item() == 0
+    assert np.all(out["inv_MK"].numpy() == -1)
+    short = mask.clone()
+    short[:, 17] = 0
+    for m in (3, 20, 39):
+        short[int(torch.nonzero(short[:, m])[-1]), m] = 0
+    out = _run(short, K)
+    o = oracle.index_build(short)
+    total = int(o["cumsums_N"][-1])
+    assert total == M * K - K - 3 and out["violations"].item() == 4
+    for k in ("sizes_N", "cumsums_N"):
+        assert np.array_equal(out[k].numpy(), o[k]), k
+    assert np.array_equal(out["idx_Msum"].numpy()[:total], o["idx_Msum"])
+    assert np.array_equal(out["which_Msum"].numpy()[:total], o["which_Msum"])
+    assert np.all(out["idx_Msum"].numpy()[total:] == 0) and np.all(out["which_Msum"].numpy()[total:] == 0)
+    assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
