@@ -208,3 +208,25 @@ def test_violations_strides_and_missing_pairs_with_one_thread_per_expert():
     assert np.array_equal(out["which_Msum"].numpy()[:total], o["which_Msum"])
     assert np.all(out["idx_Msum"].numpy()[total:] == 0) and np.all(out["which_Msum"].numpy()[total:] == 0)
     assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
+
+
+def test_random_shapes_of_the_single_launch_kernels():
+    # 40 seeded shapes with at most 256 tokens and 256 experts (one launch: one thread per expert
+    # up to 64 tokens, one per token above), routed and shared experts mixed, contiguous and
+    # transposed masks
+    from momoe_amd import _hip
+    rng = np.random.default_rng(17)
+    for case in range(40):
+        M = int(rng.integers(1, 65)) if case % 2 == 0 else int(rng.integers(65, 257))
+        N = int(rng.integers(1, 257))
+        K = int(rng.integers(1, min(N, 12) + 1))
+        Ks = int(rng.integers(0, K)) if case % 5 == 0 else 0
+        mask, _ = make_routing(M, N, K, Ks, seed=100 + case, skew=1.8 if case % 7 == 0 else None)
+        dev = mask.to("cuda:0")
+        if case % 3 == 0:
+            dev = mask.T.contiguous().to("cuda:0").T
+        out = {k: v.cpu() for k, v in _hip.index_build(dev, K).items()}
+        try:
+            _compare(mask, K, out)
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: M={M} N={N} K={K} Ks={Ks}: {e}") from e
