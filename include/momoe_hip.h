@@ -105,6 +105,10 @@ int64_t momoe_hbm_stream_probe(const void* matrix, int64_t blocks, int64_t krows
  * rows to an expert's tiles), or 0: the library
  * picks MOMOE_RECOMPUTE_TILE_ROWS or MOMOE_TILE_ROWS on the device (table[1] holds the choice);
  * momoe_tile_table_ints(M, N, K, 0) sizes the table for either.
+ * recompute_table (may be NULL; only with tile_rows = 0, MOMOE_ERR_BAD_ARG otherwise)
+ * int32[momoe_tile_table_ints(M, N, K, MOMOE_RECOMPUTE_TILE_ROWS)]: receives the table for tiles of
+ * MOMOE_RECOMPUTE_TILE_ROWS rows, which momoe_lin1_swiglu_bwd needs whatever height was chosen
+ * for the others (the same contents as momoe_tile_table_build would give, without its launch).
  * violations int32[1] += number of tokens whose pair count differs from K
  * (caller zeroes it; if the total pair count exceeds M*K the tile table is
  * emptied so later kernels touch nothing).
@@ -115,7 +119,7 @@ int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64_t stride_m
                       int64_t M, int64_t N, int64_t K,
                       int64_t* sizes_N, int32_t* cumsums_N1, int32_t* idx_Msum,
                       int32_t* which_Msum, int32_t* inv_MK,
-                      int32_t* tile_table, int tile_rows,
+                      int32_t* tile_table, int tile_rows, int32_t* recompute_table,
                       void* workspace, int64_t workspace_bytes,
                       int32_t* violations, void* stream);
 
@@ -146,7 +150,7 @@ int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n, int64_t s
                              int64_t M, int64_t N, int64_t K,
                              int64_t* sizes_N, int32_t* cumsums_N1, int32_t* idx_Msum,
                              int32_t* which_Msum, int32_t* inv_MK,
-                             int32_t* tile_table, int tile_rows,
+                             int32_t* tile_table, int tile_rows, int32_t* recompute_table,
                              int32_t* violations, void* stream);
 
 /* ---- experts forward -----------------------------------------------------

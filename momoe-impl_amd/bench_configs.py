@@ -225,7 +225,7 @@ CHART_GRID = [
 
 
 if __name__ == "__main__":
-    assert torch.cuda.is_available() and _hip.abi_version() == 2
+    assert torch.cuda.is_available() and _hip.abi_version() == 3
     if "--vendor" in sys.argv[1:]:
         vendor_gemms()
         read_stream_rate()

@@ -10,7 +10,7 @@ std::atomic<unsigned long long*> g_clock_trace{nullptr};
 unsigned long long* clock_trace_buffer() { return g_clock_trace.load(std::memory_order_relaxed); }
 }  // namespace momoe
 
-extern "C" int momoe_abi_version(void) { return 2; }
+extern "C" int momoe_abi_version(void) { return 3; }
 
 extern "C" const char* momoe_status_string(int status) {
   switch (status) {

@@ -93,8 +93,8 @@ __device__ __forceinline__ int choose_tile_rows(const int32_t* sizes, int N, int
 __global__ __launch_bounds__(1024) void index_scan_kernel(
     int32_t* __restrict__ part, int N, int NC, int64_t msum_cap,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums,
-    int32_t* __restrict__ table, int tile_rows_arg, int32_t* __restrict__ violations,
-    int32_t* __restrict__ idx, int32_t* __restrict__ which) {
+    int32_t* __restrict__ table, int tile_rows_arg, int32_t* __restrict__ table_rc,
+    int32_t* __restrict__ violations, int32_t* __restrict__ idx, int32_t* __restrict__ which) {
   __shared__ int32_t s_size[kMaxExperts];
   __shared__ int32_t s_cum[kMaxExperts];
   __shared__ int32_t s_first[kMaxExperts];
@@ -151,20 +151,50 @@ __global__ __launch_bounds__(1024) void index_scan_kernel(
     idx[r] = 0;
     which[r] = 0;
   }
-  if (s_total[0] == 0) return;
   const int tile_rows = s_total[2];
-  for (int i = t; i < N; i += 1024) {
-    const int v = s_size[i];
-    const int nt = (v + tile_rows - 1) / tile_rows;
-    const int first = s_first[i];
-    for (int k = 0; k < nt; ++k) {
-      int32_t* e = table + kTileHeader + 4 * (first + k);
-      e[0] = i;
-      e[1] = first;
-      e[2] = s_cum[i];
-      e[3] = v;
-    }
+  // the second table (tiles of the recomputing GEMM's height) is the same table when that is the
+  // height chosen; otherwise the row tiles are counted again below
+  const bool same = tile_rows == MOMOE_RECOMPUTE_TILE_ROWS;
+  if (s_total[0] == 0) {
+    if (table_rc != nullptr && t < kTileHeader) table_rc[t] = t == 1 ? MOMOE_RECOMPUTE_TILE_ROWS : 0;
+    return;
   }
+  auto write_entries = [&](int32_t* dst, int rows) {
+    for (int i = t; i < N; i += 1024) {
+      const int v = s_size[i];
+      const int nt = (v + rows - 1) / rows;
+      const int first = s_first[i];
+      for (int k = 0; k < nt; ++k) {
+        int32_t* e = dst + kTileHeader + 4 * (first + k);
+        e[0] = i;
+        e[1] = first;
+        e[2] = s_cum[i];
+        e[3] = v;
+      }
+    }
+  };
+  write_entries(table, tile_rows);
+  if (table_rc == nullptr) return;
+  if (same) {
+    write_entries(table_rc, tile_rows);
+    if (t < kTileHeader) table_rc[t] = t == 0 ? s_total[0] : t == 1 ? tile_rows : 0;
+    return;
+  }
+  __syncthreads();  // every thread has read s_first
+  if (wave == 0) {
+    int run_tiles = 0;
+    for (int i0 = 0; i0 < N; i0 += 64) {
+      const int i = i0 + lane;
+      const int v = i < N ? s_size[i] : 0;
+      const int nt = (v + MOMOE_RECOMPUTE_TILE_ROWS - 1) / MOMOE_RECOMPUTE_TILE_ROWS;
+      const int inct = wave_inclusive_scan(nt, lane);
+      if (i < N) s_first[i] = run_tiles + inct - nt;
+      run_tiles += __shfl(inct, 63);
+    }
+    if (lane < kTileHeader) table_rc[lane] = lane == 0 ? run_tiles : lane == 1 ? MOMOE_RECOMPUTE_TILE_ROWS : 0;
+  }
+  __syncthreads();
+  write_entries(table_rc, MOMOE_RECOMPUTE_TILE_ROWS);
 }
 
 __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
@@ -222,6 +252,39 @@ __global__ __launch_bounds__(kPanelTokens) void index_scatter_kernel(
 // at once: one memory latency), as 16 bits per group of 16 experts; one ballot per expert gives
 // the lane masks of its tokens, a scan over the experts gives cumsums and the tile table, and
 // every token then places its own K pairs from its bits and those masks.
+// the single-launch kernels: one expert's entries, and the header, in the table and (if asked
+// for) in its copy for the recomputing GEMM
+__device__ __forceinline__ void write_tile_entries(int32_t* table, int32_t* table_rc, int first,
+                                                   int nt, int expert, int row0, int rows) {
+  for (int k = 0; k < nt; ++k) {
+    int32_t* e = table + kTileHeader + 4 * (first + k);
+    e[0] = expert;
+    e[1] = first;
+    e[2] = row0;
+    e[3] = rows;
+    if (table_rc != nullptr) {
+      int32_t* c = table_rc + kTileHeader + 4 * (first + k);
+      c[0] = expert;
+      c[1] = first;
+      c[2] = row0;
+      c[3] = rows;
+    }
+  }
+}
+__device__ __forceinline__ void write_tile_header(int32_t* table, int32_t* table_rc, int ntiles,
+                                                  int tile_rows) {
+  table[0] = ntiles;
+  table[1] = tile_rows;
+  table[2] = 0;
+  table[3] = 0;
+  if (table_rc != nullptr) {
+    table_rc[0] = ntiles;
+    table_rc[1] = tile_rows;
+    table_rc[2] = 0;
+    table_rc[3] = 0;
+  }
+}
+
 constexpr int kSmallMaxGroups = 16;
 constexpr int kSmallMaxExperts = kSmallMaxGroups * kPanelExperts;
 
@@ -230,9 +293,9 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
     int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
-    int tile_rows_arg, int32_t* __restrict__ violations) {
+    int tile_rows_arg, int32_t* __restrict__ table_rc, int32_t* __restrict__ violations) {
   // asked to choose the tile height: with at most 256 tokens no expert holds more than 256 rows,
-  // and taller tiles save nothing
+  // and taller tiles save nothing.  table_rc (only with that choice) receives the same table.
   const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
   static_assert(kPanelTokens <= MOMOE_RECOMPUTE_TILE_ROWS, "one tile per expert in the one-launch kernel");
   __shared__ uint64_t ball[NGROUPS * kPanelExperts][4];  // tokens of expert i in wave w, as a lane mask
@@ -272,22 +335,12 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
   if (t < N) {
     cumsums[t] = brow;
     sizes[t] = (int64_t)v;
-    if (!overflow)
-      for (int k = 0; k < nt; ++k) {
-        int32_t* e = table + kTileHeader + 4 * (btile + k);
-        e[0] = t;
-        e[1] = btile;
-        e[2] = brow;
-        e[3] = v;
-      }
+    if (!overflow) write_tile_entries(table, table_rc, btile, nt, t, brow, v);
   }
   if (t == 0) {
     cumsums[N] = total;
     if (overflow) atomicAdd(violations, 1);
-    table[0] = overflow ? 0 : total_tiles;
-    table[1] = tile_rows;
-    table[2] = 0;
-    table[3] = 0;
+    write_tile_header(table, table_rc, overflow ? 0 : total_tiles, tile_rows);
   }
   // sorted rows past the last pair (a routing with fewer than M*K pairs): token 0, slot 0
   for (int64_t r = (int64_t)total + t; r < msum; r += kPanelTokens) {
@@ -332,7 +385,7 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
     int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
-    int tile_rows_arg, int32_t* __restrict__ violations) {
+    int tile_rows_arg, int32_t* __restrict__ table_rc, int32_t* __restrict__ violations) {
   static_assert(MCH >= 1 && 16 * MCH <= kTinyTokens, "token chunks of 16");
   const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
   __shared__ uint64_t tokb[kTinyTokens][4];  // experts of token m among the experts of wave w, as a lane mask
@@ -375,22 +428,12 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
   if (e < N) {
     cumsums[e] = brow;
     sizes[e] = (int64_t)v;
-    if (!overflow)
-      for (int k = 0; k < nt; ++k) {
-        int32_t* t = table + kTileHeader + 4 * (btile + k);
-        t[0] = e;
-        t[1] = btile;
-        t[2] = brow;
-        t[3] = v;
-      }
+    if (!overflow) write_tile_entries(table, table_rc, btile, nt, e, brow, v);
   }
   if (e == 0) {
     cumsums[N] = total;
     if (overflow) atomicAdd(violations, 1);
-    table[0] = overflow ? 0 : total_tiles;
-    table[1] = tile_rows;
-    table[2] = 0;
-    table[3] = 0;
+    write_tile_header(table, table_rc, overflow ? 0 : total_tiles, tile_rows);
   }
   // sorted rows past the last pair (a routing with fewer than M*K pairs): token 0, slot 0
   for (int64_t r = (int64_t)total + e; r < msum; r += kPanelTokens) {
@@ -503,14 +546,16 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
                                  int64_t M, int64_t N, int64_t K, int64_t* sizes_N,
                                  int32_t* cumsums_N1, int32_t* idx_Msum, int32_t* which_Msum,
                                  int32_t* inv_MK, int32_t* tile_table, int tile_rows,
-                                 void* workspace, int64_t workspace_bytes, int32_t* violations,
-                                 void* stream) {
+                                 int32_t* recompute_table, void* workspace,
+                                 int64_t workspace_bytes, int32_t* violations, void* stream) {
   if (!mask_NM || !sizes_N || !cumsums_N1 || !idx_Msum || !which_Msum || !inv_MK || !tile_table ||
       !workspace || !violations)
     return MOMOE_ERR_BAD_ARG;
   if (M <= 0 || N <= 0 || K <= 0 || tile_rows < 0) return MOMOE_ERR_BAD_ARG;
   if (N > kMaxExperts || M * K >= (1ll << 31) || M >= (1ll << 30)) return MOMOE_ERR_UNSUPPORTED;
   if (tile_rows != 0 && !tile_height_ok(tile_rows)) return MOMOE_ERR_UNSUPPORTED;
+  // the second table goes with the library's own choice of the height
+  if (recompute_table != nullptr && tile_rows != 0) return MOMOE_ERR_BAD_ARG;
   if (workspace_bytes < momoe_index_workspace_bytes(M, N)) return MOMOE_ERR_BAD_ARG;
   const int NC = (int)cdiv64(M, kPanelTokens), NG = (int)cdiv64(N, kPanelExperts);
   if (NG > 65535) return MOMOE_ERR_UNSUPPORTED;
@@ -522,21 +567,22 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
                 : M <= 48 ? index_tiny_kernel<3> : index_tiny_kernel<4>;
     kernel<<<1, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N,
                                        cumsums_N1, idx_Msum, which_Msum, inv_MK, tile_table,
-                                       tile_rows, violations);
+                                       tile_rows, recompute_table, violations);
     return launch_status();
   }
   if (NC == 1 && N <= kSmallMaxExperts) {
     auto kernel = N <= 128 ? index_small_kernel<8> : index_small_kernel<kSmallMaxGroups>;
     kernel<<<1, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N,
                                        cumsums_N1, idx_Msum, which_Msum, inv_MK, tile_table,
-                                       tile_rows, violations);
+                                       tile_rows, recompute_table, violations);
     return launch_status();
   }
   dim3 grid(NC, NG);
   index_count_kernel<<<grid, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N,
                                                     NC, part, tokcnt);
   index_scan_kernel<<<1, 1024, 0, st>>>(part, (int)N, NC, M * K, sizes_N, cumsums_N1, tile_table,
-                                        tile_rows, violations, idx_Msum, which_Msum);
+                                        tile_rows, recompute_table, violations, idx_Msum,
+                                        which_Msum);
   index_scatter_kernel<<<grid, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N,
                                                       (int)K, NC, part, tokcnt, cumsums_N1,
                                                       idx_Msum, which_Msum, inv_MK, violations);
@@ -577,7 +623,8 @@ extern "C" int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n
                                         int64_t M, int64_t N, int64_t K, int64_t* sizes_N,
                                         int32_t* cumsums_N1, int32_t* idx_Msum,
                                         int32_t* which_Msum, int32_t* inv_MK, int32_t* tile_table,
-                                        int tile_rows, int32_t* violations, void* stream) {
+                                        int tile_rows, int32_t* recompute_table,
+                                        int32_t* violations, void* stream) {
   if (M <= 0 || N <= 0) return MOMOE_ERR_BAD_ARG;
   // sizes beyond the fixed array are refused, never truncated
   if (momoe_index_workspace_bytes(M, N) > kStaticScratchBytes) return MOMOE_ERR_UNSUPPORTED;
@@ -587,6 +634,6 @@ extern "C" int momoe_index_build_static(const int32_t* mask_NM, int64_t stride_n
   // Every word of the array that the scatter pass reads was written by the count pass of the
   // same call, so nothing has to be cleared between calls.
   return momoe_index_build(mask_NM, stride_n, stride_m, M, N, K, sizes_N, cumsums_N1, idx_Msum,
-                           which_Msum, inv_MK, tile_table, tile_rows, ws, kStaticScratchBytes,
-                           violations, stream);
+                           which_Msum, inv_MK, tile_table, tile_rows, recompute_table, ws,
+                           kStaticScratchBytes, violations, stream);
 }

@@ -38,10 +38,10 @@ _SIGNATURES = {
     "momoe_tile_table_ints": (_i64, [_i64, _i64, _i64, _int]),
     "momoe_index_workspace_bytes": (_i64, [_i64, _i64]),
     "momoe_index_build": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _int,
-                                 _p, _i64, _p, _p]),
+                                 _p, _p, _i64, _p, _p]),
     "momoe_tile_table_build": (_int, [_p, _i64, _i64, _int, _p, _p]),
     "momoe_index_build_static": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p,
-                                        _int, _p, _p]),
+                                        _int, _p, _p, _p]),
     "momoe_lin1_swiglu_fwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64,
                                      _i64, _p]),
     "momoe_lin2_scale_fwd": (_int, [_p, _p, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64,
@@ -198,10 +198,12 @@ def abi_version():
 
 
 # ---------------------------------------------------------------- index build
-def index_build(mask_NM, K, static_scratch=False, tile_rows=AUTO_TILE_ROWS):
+def index_build(mask_NM, K, static_scratch=False, tile_rows=AUTO_TILE_ROWS, recompute_table=False):
     """mask_NM int32 [N,M] (any strides) -> dict of device tensors.
     See momoe_index_build in include/momoe_hip.h.  static_scratch=True goes through
-    momoe_index_build_static: no workspace is allocated, the library's fixed array is used."""
+    momoe_index_build_static: no workspace is allocated, the library's fixed array is used.
+    recompute_table=True (only with tile_rows=AUTO_TILE_ROWS) also returns "recompute_table", the
+    table of RECOMPUTE_TILE_ROWS-row tiles that lin1_swiglu_bwd walks."""
     _need_cuda(mask_NM)
     assert mask_NM.dtype == torch.int32 and mask_NM.dim() == 2
     N, M = mask_NM.shape
@@ -213,19 +215,26 @@ def index_build(mask_NM, K, static_scratch=False, tile_rows=AUTO_TILE_ROWS):
     which = torch.empty(msum, dtype=torch.int32, device=dev)
     inv = torch.empty(msum, dtype=torch.int32, device=dev)
     table = torch.empty(_lib.momoe_tile_table_ints(M, N, K, tile_rows), dtype=torch.int32, device=dev)
+    table_rc = None
+    if recompute_table:
+        table_rc = torch.empty(_lib.momoe_tile_table_ints(M, N, K, RECOMPUTE_TILE_ROWS), dtype=torch.int32,
+                               device=dev)
     violations = torch.zeros(1, dtype=torch.int32, device=dev)
     if static_scratch:
         _call("momoe_index_build_static", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N,
               K, _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv), _ptr(table),
-              tile_rows, _ptr(violations), _stream())
+              tile_rows, _ptr(table_rc), _ptr(violations), _stream())
     else:
         ws_bytes = _lib.momoe_index_workspace_bytes(M, N)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         _call("momoe_index_build", _ptr(mask_NM), mask_NM.stride(0), mask_NM.stride(1), M, N, K,
               _ptr(sizes), _ptr(cumsums), _ptr(idx), _ptr(which), _ptr(inv), _ptr(table),
-              tile_rows, _ptr(ws), ws_bytes, _ptr(violations), _stream())
-    return {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
-            "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
+              tile_rows, _ptr(table_rc), _ptr(ws), ws_bytes, _ptr(violations), _stream())
+    out = {"sizes_N": sizes, "cumsums_N": cumsums, "idx_Msum": idx, "which_Msum": which,
+           "inv_MK": inv.view(M, K), "tile_table": table, "violations": violations}
+    if table_rc is not None:
+        out["recompute_table"] = table_rc
+    return out
 
 
 def tile_table_build(cumsums_N1, M, K, tile_rows):

@@ -78,10 +78,13 @@ class MoEFunction(torch.autograd.Function):
             if ctx.needs_input_grad[1] and 8 * msum * 64 >= 2 ** 32:
                 raise RuntimeError(f"MoMoE backward supports fewer than 8388608 (token, expert) pairs per call, "
                                    f"got {msum}: split the batch")
-            ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS)
-            idx, table = ib["idx_Msum"], ib["tile_table"]
             # nothing is kept for a backward that cannot happen (no input wants a gradient)
             msave = _saved_rows(msum, save_percent) if any(ctx.needs_input_grad[:5]) else 0
+            # the backward's recomputing GEMM walks row tiles of its own height: with the height
+            # left to the library, the index build writes that table too
+            want_rc = any(ctx.needs_input_grad[:5]) and msave < msum and TILE_ROWS == _hip.AUTO_TILE_ROWS
+            ib = _hip.index_build(mask, K, tile_rows=TILE_ROWS, recompute_table=want_rc)
+            idx, table = ib["idx_Msum"], ib["tile_table"]
 
             # h in blocks of 32 hidden columns, [H/32][Msum][32]: the layout the down projection reads
             h = torch.empty((H // 32, msum, 32), device=dev, dtype=torch.bfloat16)
@@ -97,9 +100,12 @@ class MoEFunction(torch.autograd.Function):
         ctx.K = K
         ctx.msave = msave
         ctx.has_save = ab_save is not None
+        ctx.has_table_rc = want_rc
         saved = [x_MD, s, idx, ib["inv_MK"], ib["cumsums_N"], table, W1, W2]
         if ab_save is not None:
             saved.append(ab_save)
+        if want_rc:
+            saved.append(ib["recompute_table"])
         ctx.save_for_backward(*saved)
         if CHECK_ROUTING and int(ib["violations"].item()) != 0:
             raise RuntimeError(f"mask_NM: {int(ib['violations'].item())} tokens do not have exactly K = {K} "
@@ -113,6 +119,7 @@ class MoEFunction(torch.autograd.Function):
         saved = ctx.saved_tensors
         x_MD, s, idx, inv, cumsums, table, W1, W2 = saved[:8]
         ab_save = saved[8] if ctx.has_save else None
+        table_rc = saved[-1] if ctx.has_table_rc else None
         msave = ctx.msave
         B, S, D = G_y_BSD.shape
         M = B * S
@@ -139,8 +146,10 @@ class MoEFunction(torch.autograd.Function):
             if msave > 0:
                 _hip.swiglu_bwd_saved(ab_save, u, s, idx, cumsums, msave, gz, hsT, gs_part)
             if msave < msum:
-                # the recomputing GEMM takes shorter row tiles than the others: its own table
-                table_rc = _hip.tile_table_build(cumsums, M, ctx.K, _hip.RECOMPUTE_TILE_ROWS)
+                # the recomputing GEMM takes shorter row tiles than the others: its own table,
+                # from the index build, or made here when the tile height was given
+                if table_rc is None:
+                    table_rc = _hip.tile_table_build(cumsums, M, ctx.K, _hip.RECOMPUTE_TILE_ROWS)
                 _hip.lin1_swiglu_bwd(x_MD, W1, idx, table_rc, u, s, msave, gz, hsT, gs_part)
                 del table_rc
             del u

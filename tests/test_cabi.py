@@ -36,7 +36,7 @@ def test_every_declared_symbol_is_exported(lib):
 def test_binding_table_matches_header():
     from momoe_amd import _hip
     assert sorted(_hip.EXPORTED_SYMBOLS) == _declared()
-    assert _hip.abi_version() == 2
+    assert _hip.abi_version() == 3
     assert _hip.status_string(0) == "ok" and "unsupported" in _hip.status_string(2)
 
 

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 def _run(mask, K):
     from momoe_amd import _hip
-    out = _hip.index_build(mask.to("cuda:0"), K)
+    out = _hip.index_build(mask.to("cuda:0"), K, recompute_table=True)
     torch.cuda.synchronize()
     return {k: v.cpu() for k, v in out.items()}
 
@@ -43,6 +43,9 @@ def _compare(mask, K, out):
         return sum(int(v) + 256 * -(-int(v) // rows) for v in o["sizes_N"])
     tall = cost(_hip.TILE_ROWS) * 26 < cost(_hip.RECOMPUTE_TILE_ROWS) * 25
     _check_table(out["tile_table"].numpy(), o, _hip.TILE_ROWS if tall else _hip.RECOMPUTE_TILE_ROWS)
+    # the recomputing GEMM's table, written by the same call when asked for
+    if "recompute_table" in out:
+        _check_table(out["recompute_table"].numpy(), o, _hip.RECOMPUTE_TILE_ROWS)
     # the table for another tile height, made from the prefix sums alone
     M = mask.shape[1]
     for rows in (_hip.RECOMPUTE_TILE_ROWS, _hip.TILE_ROWS, 32):
@@ -92,6 +95,9 @@ def test_index_with_a_given_tile_height():
 def test_tile_heights_no_kernel_takes_are_refused():
     from momoe_amd import _hip
     mask, _ = make_routing(300, 8, 2, seed=1)
+    # the second table comes with the library's own choice of the height only
+    with pytest.raises(RuntimeError):
+        _hip.index_build(mask.to("cuda:0"), 2, tile_rows=_hip.RECOMPUTE_TILE_ROWS, recompute_table=True)
     with pytest.raises(RuntimeError):
         _hip.index_build(mask.to("cuda:0"), 2, tile_rows=_hip.TILE_ROWS + 32)
     ib = _hip.index_build(mask.to("cuda:0"), 2)
@@ -121,6 +127,11 @@ def test_violation_counter_and_no_out_of_bounds():
     bad[0:6, 9] = 1        # token 9 has more than K
     out = _run(bad, 4)
     assert out["violations"].item() >= 2
+    # too many pairs in total: both tile tables are emptied
+    out = _run(torch.ones(16, 512, dtype=torch.int32), 4)
+    assert out["violations"].item() >= 1
+    assert out["tile_table"][0].item() == 0 and out["recompute_table"][0].item() == 0
+    assert out["recompute_table"][1].item() == 256
 
 
 def test_violations_single_panel():
@@ -134,6 +145,7 @@ def test_violations_single_panel():
     over = torch.ones(40, 100, dtype=torch.int32)
     out = _run(over, 4)
     assert out["violations"].item() >= 1 and out["tile_table"][0].item() == 0
+    assert out["recompute_table"][0].item() == 0
     # a table made from those prefix sums is empty as well
     from momoe_amd import _hip
     t = _hip.tile_table_build(out["cumsums_N"].to("cuda:0"), 100, 4, _hip.RECOMPUTE_TILE_ROWS)
@@ -225,7 +237,7 @@ def test_random_shapes_of_the_single_launch_kernels():
         dev = mask.to("cuda:0")
         if case % 3 == 0:
             dev = mask.T.contiguous().to("cuda:0").T
-        out = {k: v.cpu() for k, v in _hip.index_build(dev, K).items()}
+        out = {k: v.cpu() for k, v in _hip.index_build(dev, K, recompute_table=case % 4 != 1).items()}
         try:
             _compare(mask, K, out)
         except AssertionError as e:

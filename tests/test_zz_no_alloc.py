@@ -42,7 +42,7 @@ def test_static_scratch_allocates_nothing_and_refuses_oversized_inputs():
     d = mask.to("cuda:0")
     _hip.index_build(d, K, static_scratch=True)  # first call on the device: address look-up
     torch.cuda.synchronize()
-    out = {k: torch.empty_like(v) for k, v in _hip.index_build(d, K).items()}
+    out = {k: torch.empty_like(v) for k, v in _hip.index_build(d, K, recompute_table=True).items()}
     out["violations"].zero_()
     torch.cuda.synchronize()
     free_before, _ = torch.cuda.mem_get_info()
@@ -50,19 +50,21 @@ def test_static_scratch_allocates_nothing_and_refuses_oversized_inputs():
         d.data_ptr(), d.stride(0), d.stride(1), M, N, K, out["sizes_N"].data_ptr(),
         out["cumsums_N"].data_ptr(), out["idx_Msum"].data_ptr(), out["which_Msum"].data_ptr(),
         out["inv_MK"].data_ptr(), out["tile_table"].data_ptr(), _hip.AUTO_TILE_ROWS,
-        out["violations"].data_ptr(), torch.cuda.current_stream().cuda_stream)
+        out["recompute_table"].data_ptr(), out["violations"].data_ptr(),
+        torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     free_after, _ = torch.cuda.mem_get_info()
     assert rc == 0 and free_after == free_before  # no device memory was taken from the driver
-    ref = _hip.index_build(d, K)
+    ref = _hip.index_build(d, K, recompute_table=True)
     torch.cuda.synchronize()
     for k in ("sizes_N", "cumsums_N", "idx_Msum", "which_Msum", "inv_MK"):
         assert torch.equal(out[k], ref[k]), k
-    used = 4 + 4 * int(ref["tile_table"][0])
-    assert torch.equal(out["tile_table"][:used], ref["tile_table"][:used])
+    for k in ("tile_table", "recompute_table"):
+        used = 4 + 4 * int(ref[k][0])
+        assert torch.equal(out[k][:used], ref[k][:used]), k
     # 65536 tokens x 256 experts needs 4.2 MiB of panel counts: more than the fixed array
     z = ctypes.c_void_p(0)
     i64 = ctypes.c_int64
     assert _hip._lib.momoe_index_workspace_bytes(65536, 256) > 4 * 2**20
     assert _hip._lib.momoe_index_build_static(z, i64(1), i64(1), i64(65536), i64(256), i64(8), z, z, z, z,
-                                              z, z, 256, z, z) == 2
+                                              z, z, 256, z, z, z) == 2
