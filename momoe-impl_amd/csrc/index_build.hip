@@ -299,8 +299,9 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
   const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
   static_assert(kPanelTokens <= MOMOE_RECOMPUTE_TILE_ROWS, "one tile per expert in the one-launch kernel");
   __shared__ uint64_t ball[NGROUPS * kPanelExperts][4];  // tokens of expert i in wave w, as a lane mask
-  __shared__ int32_t s_cum[NGROUPS * kPanelExperts];
+  __shared__ int32_t s_base[NGROUPS * kPanelExperts][4];  // sorted row of expert i's first token in wave w
   __shared__ int32_t s_wave[4][2];
+  static_assert(NGROUPS % 4 == 0, "the experts of a token are walked as 64-bit words");
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int64_t msum = (int64_t)M * K;
   uint32_t bits[NGROUPS];
@@ -331,8 +332,13 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
   const int total = s_wave[0][0] + s_wave[1][0] + s_wave[2][0] + s_wave[3][0];
   const int total_tiles = s_wave[0][1] + s_wave[1][1] + s_wave[2][1] + s_wave[3][1];
   const bool overflow = (int64_t)total > msum;
-  if (t < NGROUPS * kPanelExperts) s_cum[t] = brow;
   if (t < N) {
+    int run = brow;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      s_base[t][w] = run;
+      run += __popcll(ball[t][w]);
+    }
     cumsums[t] = brow;
     sizes[t] = (int64_t)v;
     if (!overflow) write_tile_entries(table, table_rc, btile, nt, t, brow, v);
@@ -348,25 +354,33 @@ __global__ __launch_bounds__(kPanelTokens) void index_small_kernel(
     which[r] = 0;
   }
   __syncthreads();
-  // every token walks its own pairs (K of them, not N candidates), lowest expert first
+  // every token walks its own pairs (K of them, not N candidates), lowest expert first: one loop
+  // over all of its experts, so that a wavefront makes as many rounds as its busiest token has
+  // pairs (a loop per group of 16 experts made the sum over the groups of that maximum)
   const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  int k = 0;
+  constexpr int NWORDS = NGROUPS / 4;
+  uint64_t word[NWORDS];
 #pragma unroll
-  for (int g = 0; g < NGROUPS; ++g) {
-    uint32_t rest = bits[g];
-    while (rest != 0) {
-      const int i = g * kPanelExperts + __ffs(rest) - 1;
-      rest &= rest - 1;
-      int before = __popcll(ball[i][wave] & below);
-      for (int w = 0; w < wave; ++w) before += __popcll(ball[i][w]);
-      const int64_t row = (int64_t)s_cum[i] + before;
-      if (row < msum) {
-        idx[row] = t;
-        which[row] = k;
-      }
-      if (k < K) inv[(int64_t)t * K + k] = row < msum && !overflow ? (int32_t)row : -1;
-      ++k;
+  for (int j = 0; j < NWORDS; ++j)
+    word[j] = (uint64_t)bits[4 * j] | ((uint64_t)bits[4 * j + 1] << 16) |
+              ((uint64_t)bits[4 * j + 2] << 32) | ((uint64_t)bits[4 * j + 3] << 48);
+  int k = 0;
+  for (;;) {
+    int i = -1;
+#pragma unroll
+    for (int j = NWORDS - 1; j >= 0; --j)
+      if (word[j] != 0) i = 64 * j + __ffsll((unsigned long long)word[j]) - 1;
+    if (i < 0) break;
+#pragma unroll
+    for (int j = 0; j < NWORDS; ++j)
+      if ((i >> 6) == j) word[j] &= word[j] - 1;
+    const int64_t row = (int64_t)s_base[i][wave] + __popcll(ball[i][wave] & below);
+    if (row < msum) {
+      idx[row] = t;
+      which[row] = k;
     }
+    if (k < K) inv[(int64_t)t * K + k] = row < msum && !overflow ? (int32_t)row : -1;
+    ++k;
   }
   if (t < M && k != K) {
     atomicAdd(violations, 1);
@@ -389,6 +403,7 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
   static_assert(MCH >= 1 && 16 * MCH <= kTinyTokens, "token chunks of 16");
   const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
   __shared__ uint64_t tokb[kTinyTokens][4];  // experts of token m among the experts of wave w, as a lane mask
+  __shared__ int32_t s_slot[kTinyTokens][4];  // pairs of token m held by the experts of the waves below w
   __shared__ int32_t s_wave[4][2];
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
   const int64_t msum = (int64_t)M * K;
@@ -440,6 +455,16 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
     idx[r] = 0;
     which[r] = 0;
   }
+  // thread m counts the pairs of token m
+  int pairs = 0;
+  if (e < M) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      s_slot[e][w] = pairs;
+      pairs += __popcll(tokb[e][w]);
+    }
+  }
+  __syncthreads();
   // the expert places its pairs, lowest token first; the slot of a pair within its token is the
   // number of lower-numbered experts that hold the token
   const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
@@ -447,8 +472,7 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
   for (int r = 0; rest != 0; ++r) {
     const int m = __ffsll((unsigned long long)rest) - 1;
     rest &= rest - 1;
-    int k = __popcll(tokb[m][wave] & below);
-    for (int w = 0; w < wave; ++w) k += __popcll(tokb[m][w]);
+    const int k = s_slot[m][wave] + __popcll(tokb[m][wave] & below);
     const int64_t srow = (int64_t)brow + r;
     if (srow < msum) {
       idx[srow] = m;
@@ -457,12 +481,9 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
     if (k < K) inv[(int64_t)m * K + k] = srow < msum && !overflow ? (int32_t)srow : -1;
   }
   // tokens whose pair count is not K: thread m looks after token m
-  if (e < M) {
-    const int k = __popcll(tokb[e][0]) + __popcll(tokb[e][1]) + __popcll(tokb[e][2]) + __popcll(tokb[e][3]);
-    if (k != K) {
-      atomicAdd(violations, 1);
-      for (int kk = k; kk < K; ++kk) inv[(int64_t)e * K + kk] = -1;
-    }
+  if (e < M && pairs != K) {
+    atomicAdd(violations, 1);
+    for (int kk = pairs; kk < K; ++kk) inv[(int64_t)e * K + kk] = -1;
   }
 }
 
