@@ -400,7 +400,8 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
     const int32_t* __restrict__ mask, int64_t sn, int64_t sm, int M, int N, int K,
     int64_t* __restrict__ sizes, int32_t* __restrict__ cumsums, int32_t* __restrict__ idx,
     int32_t* __restrict__ which, int32_t* __restrict__ inv, int32_t* __restrict__ table,
-    int tile_rows_arg, int32_t* __restrict__ table_rc, int32_t* __restrict__ violations) {
+    int tile_rows_arg, int32_t* __restrict__ table_rc, int32_t* __restrict__ violations,
+    bool rows_of_int4) {
   static_assert(MCH >= 1 && 16 * MCH <= kTinyTokens, "token chunks of 16");
   const int tile_rows = tile_rows_arg > 0 ? tile_rows_arg : MOMOE_RECOMPUTE_TILE_ROWS;
   __shared__ uint64_t tokb[kTinyTokens][4];  // experts of token m among the experts of wave w, as a lane mask
@@ -410,15 +411,28 @@ __global__ __launch_bounds__(kPanelTokens) void index_tiny_kernel(
   const int64_t msum = (int64_t)M * K;
   // the expert's row of the mask as a bit set; loads unconditional, row and column clamped
   uint64_t bits = 0;
-  {
-    const int32_t* row = mask + (int64_t)min(e, N - 1) * sn;
+  const int32_t* row = mask + (int64_t)min(e, N - 1) * sn;
+  if (rows_of_int4) {
+    // contiguous rows of a multiple of 4 tokens, 16-byte aligned (checked on the host): four
+    // tokens per load.  Lanes read rows that lie apart, so a load instruction costs one line
+    // request per lane whatever its width, and this path makes a quarter of them.
+    int4 v[4 * MCH];
+#pragma unroll
+    for (int c = 0; c < 4 * MCH; ++c) v[c] = ((const int4*)row)[min(c, M / 4 - 1)];
+#pragma unroll
+    for (int c = 0; c < 4 * MCH; ++c) {
+      const uint64_t nib = (v[c].x != 0 ? 1u : 0u) | (v[c].y != 0 ? 2u : 0u) | (v[c].z != 0 ? 4u : 0u) |
+                           (v[c].w != 0 ? 8u : 0u);
+      if (4 * c < M) bits |= nib << (4 * c);
+    }
+  } else {
     int32_t v[16 * MCH];
 #pragma unroll
     for (int m = 0; m < 16 * MCH; ++m) v[m] = row[(int64_t)min(m, M - 1) * sm];
 #pragma unroll
     for (int m = 0; m < 16 * MCH; ++m) bits |= (uint64_t)(v[m] != 0 && m < M ? 1 : 0) << m;
-    if (e >= N) bits = 0;
   }
+  if (e >= N) bits = 0;
   // per token: the experts that hold it
   for (int m = 0; m < M; ++m) {
     const uint64_t b = __ballot((bits >> m) & 1ull);
@@ -587,9 +601,10 @@ extern "C" int momoe_index_build(const int32_t* mask_NM, int64_t stride_n, int64
   if (M <= kTinyTokens && N <= kPanelTokens) {
     auto kernel = M <= 16 ? index_tiny_kernel<1> : M <= 32 ? index_tiny_kernel<2>
                 : M <= 48 ? index_tiny_kernel<3> : index_tiny_kernel<4>;
+    const bool rows_of_int4 = stride_m == 1 && stride_n % 4 == 0 && M % 4 == 0 && ((uintptr_t)mask_NM & 15) == 0;
     kernel<<<1, kPanelTokens, 0, st>>>(mask_NM, stride_n, stride_m, (int)M, (int)N, (int)K, sizes_N,
                                        cumsums_N1, idx_Msum, which_Msum, inv_MK, tile_table,
-                                       tile_rows, recompute_table, violations);
+                                       tile_rows, recompute_table, violations, rows_of_int4);
     return launch_status();
   }
   if (NC == 1 && N <= kSmallMaxExperts) {

@@ -197,6 +197,15 @@ def test_violations_strides_and_missing_pairs_with_one_thread_per_expert():
     mask, _ = make_routing(M, N, K, seed=5)
     strided = mask.T.contiguous().to("cuda:0").T  # strides (1, N)
     _compare(mask, K, {k: v.cpu() for k, v in _hip.index_build(strided, K).items()})
+    # views into a wider matrix: rows that start 16 bytes / 4 bytes into a line (the kernel reads
+    # aligned rows of a multiple of four tokens with 16-byte loads, anything else entry by entry)
+    wide = torch.zeros(N, M + 8, dtype=torch.int32)
+    for first in (4, 1):
+        wide.zero_()
+        wide[:, first:first + M] = mask
+        view = wide.to("cuda:0")[:, first:first + M]
+        assert not view.is_contiguous()
+        _compare(mask, K, {k: v.cpu() for k, v in _hip.index_build(view, K).items()})
     bad = mask.clone()
     bad[:, 5] = 0          # token 5 has no expert
     bad[0:6, 9] = 1        # token 9 has more than K
