@@ -76,6 +76,11 @@ def _compare(mask, K, out):
     (17, 255, 6, 0, 1.8),       # skewed, one token past a chunk of 16
     (64, 257, 4, 0, None),      # one expert too many for it: the one-panel kernel
     (65, 256, 4, 0, None),      # one token too many
+    # a few token panels
+    (1024, 128, 8, 0, None),
+    (257, 1, 1, 0, None),       # a single expert: one 320-row tile, two of 256 rows for the recomputing GEMM
+    (1024, 64, 8, 4, 1.8),      # experts of up to 1024 rows: tall tiles chosen on the device
+    (700, 128, 8, 0, 1.8),
 ])
 def test_index_bit_exact(M, N, K, Ks, skew):
     mask, _ = make_routing(M, N, K, Ks, seed=11, skew=skew)
@@ -231,20 +236,20 @@ def test_violations_strides_and_missing_pairs_with_one_thread_per_expert():
     assert np.array_equal(out["inv_MK"].numpy(), o["inv_MK"])
 
 
-def test_random_shapes_of_the_single_launch_kernels():
-    # 40 seeded shapes with at most 256 tokens and 256 experts (one launch: one thread per expert
-    # up to 64 tokens, one per token above), routed and shared experts mixed, contiguous and
-    # transposed masks
+def test_random_shapes_up_to_1024_tokens():
+    # 60 seeded shapes: the single-launch kernels (one thread per expert up to 64 tokens, one per
+    # token up to 256 tokens and 256 experts) and a few token panels, routed and shared experts
+    # mixed, contiguous and transposed masks
     from momoe_amd import _hip
     rng = np.random.default_rng(17)
-    for case in range(40):
-        M = int(rng.integers(1, 65)) if case % 2 == 0 else int(rng.integers(65, 257))
-        N = int(rng.integers(1, 257))
+    for case in range(60):
+        M = int(rng.integers(1, 65)) if case % 3 == 0 else int(rng.integers(65, 257)) if case % 3 == 1 else int(rng.integers(257, 1025))
+        N = int(rng.integers(1, 257)) if M <= 256 else int(rng.integers(1, 129))
         K = int(rng.integers(1, min(N, 12) + 1))
         Ks = int(rng.integers(0, K)) if case % 5 == 0 else 0
         mask, _ = make_routing(M, N, K, Ks, seed=100 + case, skew=1.8 if case % 7 == 0 else None)
         dev = mask.to("cuda:0")
-        if case % 3 == 0:
+        if case % 4 == 0:
             dev = mask.T.contiguous().to("cuda:0").T
         out = {k: v.cpu() for k, v in _hip.index_build(dev, K, recompute_table=case % 4 != 1).items()}
         try:
